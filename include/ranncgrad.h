@@ -1,0 +1,163 @@
+/*
+ * libranncgrad -- C ABI of the MI355X (gfx950) kernel library for the per-step
+ * parameter/gradient path of RaNNC: pack gradients into buckets, loss-scale
+ * unscale with an inf/NaN flag, global L2 norm + clip-by-norm, master-parameter
+ * casts, and flat-buffer <-> segment copies.
+ *
+ * Conventions
+ *  - every entry point returns an int status (RG_OK == 0); none throws;
+ *    rg_last_error() gives the message of the calling thread's last failure;
+ *  - pointers named *_dev / src / dst are device pointers owned by the caller and
+ *    borrowed for the duration of the call (plans keep them until updated);
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *    all device work is enqueued on it and nothing synchronises with the host
+ *    except rg_plan_create / rg_plan_destroy / rg_read_* ;
+ *  - after rg_plan_create no entry point allocates device memory.
+ *
+ * The reference has no GPU kernels for this path: it issues one ATen op per
+ * tensor from C++ loops.  Each declaration cites the reference code it replaces
+ * (paths relative to the reference tree).
+ */
+#ifndef RANNCGRAD_H
+#define RANNCGRAD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RG_VERSION 1
+
+/* status codes */
+enum {
+  RG_OK = 0,
+  RG_EINVAL = 1, /* bad argument (reference: std::invalid_argument -> ValueError) */
+  RG_EALIGN = 2, /* pointer not aligned to its element size */
+  RG_EHIP = 3,   /* a HIP runtime call failed (reference: std::runtime_error)  */
+  RG_ENOMEM = 4
+};
+
+/* element types; the reference admits exactly these three
+ * (assert at src/comp/ParamStorage.cpp:51-53) */
+enum { RG_F32 = 0, RG_F16 = 1, RG_BF16 = 2 };
+
+/* flags for rg_fused_step */
+enum {
+  RG_STEP_DEFAULT = 0,
+  /* On overflow still write the unscaled (unclipped) values, as Apex's
+   * multi_tensor_scale does; by default the write pass is skipped because the
+   * step is skipped and the gradients are discarded. */
+  RG_STEP_WRITE_ON_OVERFLOW = 1,
+  /* Report the flag but let it gate nothing: a non-finite norm then behaves exactly as in
+   * ParamStorage::clipGradNorm (inf -> coef 0, NaN -> no clip; src/comp/ParamStorage.cpp:723-742).
+   * This is what RaNNCModule.clip_grad_norm on existing gradients uses. */
+  RG_STEP_IGNORE_OVERFLOW = 2
+};
+
+const char* rg_last_error(void);
+int rg_version(void);
+int rg_elem_size(int dtype); /* 4, 2, 2; -1 for an unknown dtype */
+
+/* ---------------------------------------------------------------- layout (host only) */
+
+/* calcAlignedNumElems, src/torch/TorchUtil.cpp:1579-1591: numel rounded up to a
+ * multiple of (16 / elem_size) * split_num.  Returns -1 on bad arguments. */
+int64_t rg_aligned_numel(int64_t numel, int elem_size, int split_num);
+
+/* DistributedParamLocatorBase::doRegister, src/comp/DistributedParamLocatorBase.cpp:14-27.
+ * offsets/src_sizes receive nranks entries each. */
+int rg_segment_layout(int64_t numel, int elem_size, int nranks, int64_t* aligned_size,
+                      int64_t* segment_size, int64_t* offsets, int64_t* src_sizes);
+
+/* GradConsolidation constructor, src/comp/ParamStorage.cpp:48-57: element offset of
+ * each tensor inside the bucket of its dtype (running sum, no padding).
+ * bucket_lengths[3] is indexed by RG_F32 / RG_F16 / RG_BF16. */
+int rg_bucket_layout(int n, const int64_t* numels, const int* dtypes, int64_t* offsets,
+                     int64_t bucket_lengths[3]);
+
+/* ---------------------------------------------------------------- plans */
+
+/* A plan is a device-resident descriptor table: n tensors, each with a source
+ * pointer, a destination pointer, an element count and the two element types,
+ * cut into fixed-size chunks so that one launch covers all of them.  It replaces
+ * the reference's host loops over parameters (`for (long pid : param_ids_)`,
+ * src/comp/ParamStorage.cpp:135, 470, 726, 755).
+ *
+ * src[i] == NULL means "tensor i has no gradient": it reads as zeros
+ * (src/comp/ParamStorage.cpp:169-175).  dst[i] may be NULL only for plans that
+ * are used with rg_grad_norm alone.  dst[i] == src[i] (same dtype) is allowed:
+ * every op is then in place. */
+typedef struct rg_plan rg_plan;
+
+/* chunk_elems: elements per work chunk (multiple of 2048), 0 = choose from the total size. */
+int rg_plan_create(rg_plan** out, int device, int n, const void* const* src, void* const* dst,
+                   const int64_t* numel, const int* src_dtype, const int* dst_dtype,
+                   int64_t chunk_elems);
+/* Replace the pointers (either array may be NULL = keep); stream ordered. */
+int rg_plan_update_pointers(rg_plan* plan, const void* const* src, void* const* dst, void* stream);
+int rg_plan_destroy(rg_plan* plan);
+int rg_plan_num_tensors(const rg_plan* plan);
+int64_t rg_plan_num_chunks(const rg_plan* plan);
+int64_t rg_plan_chunk_elems(const rg_plan* plan);
+int64_t rg_plan_total_numel(const rg_plan* plan);
+
+/* ---------------------------------------------------------------- per-step operations */
+
+typedef struct rg_step_result {
+  double norm;      /* global L2 norm, as calc_grad_norm returns it (double) */
+  float coef;       /* float(max_norm / (norm + 1e-6)) when clipped, else 1 */
+  int32_t overflow; /* 1 iff any source element was +-inf or NaN */
+  int32_t clipped;  /* 1 iff the clip multiply was applied */
+  int32_t skipped;  /* 1 iff overflow gated the step (no clip; write pass skipped unless
+                       RG_STEP_WRITE_ON_OVERFLOW) */
+} rg_step_result;
+
+/* The fused step, all on the stream, no host round trip:
+ *   pass 1  read src: v = round_dst(float(x) * inv_scale); per-tensor sum v^2; inf/NaN flag
+ *   final   n_t = float(sqrt(sum_t)); norm = sqrt(sum_t double(n_t)^2) in table order;
+ *           g = norm + 1e-6; clipped = (g > max_norm) && !skipped; coef = float(max_norm / g)
+ *   pass 2  re-read src, write dst = clipped ? round_dst(v * coef) : v
+ * Replaces: Apex multi_tensor_scale (unscale + overflow flag; caller test/common.py:98-101),
+ * GradConsolidation::consolidate copy_ (src/comp/ParamStorage.cpp:159-167),
+ * ParamStorage::calcGradGlobalL2Norm (:747-819) and ParamStorage::clipGradNorm (:721-745).
+ * With dst == src and inv_scale == 1 it is exactly clip_grad_norm on existing gradients
+ * (RaNNCModule.clip_grad_norm, src/main.cpp:339-342).
+ * max_norm <= 0 disables clipping (dst = v). */
+int rg_fused_step(rg_plan* plan, float inv_scale, float max_norm, int flags, void* stream);
+
+/* One pass: dst = round_dst(float(x) * inv_scale), overflow flag and norm as above, no
+ * clip.  Apex multi_tensor_scale semantics (LossScaler.unscale). */
+int rg_unscale_pack(rg_plan* plan, float inv_scale, void* stream);
+
+/* Read-only: per-tensor and global L2 norm of the SOURCE tensors and their inf/NaN flag.
+ * ParamStorage::calcGradGlobalL2Norm, src/comp/ParamStorage.cpp:747-819
+ * (RaNNCModule.calc_grad_norm, src/main.cpp:344-345). */
+int rg_grad_norm(rg_plan* plan, void* stream);
+
+/* dst = round_dst(float(src) * scale).  scale == 1 with equal dtypes is a raw copy.
+ * Replaces per-tensor copy_/to/mul_: src/comp/ParamStorage.cpp:165, 493, 424-426, 609-611,
+ * src/comp/DistributedParamLocator.cpp:33-34, 62-65, 76,
+ * src/comp/DistributedGradLocator.cpp:59, DistributedParamLocatorBase.cpp:130-131,
+ * and Apex's master<->model copies. */
+int rg_scale_cast(rg_plan* plan, float scale, void* stream);
+
+/* dst = 0 for every tensor.  ParamStorage::clearParamGrads, src/comp/ParamStorage.cpp:540-557. */
+int rg_zero(rg_plan* plan, void* stream);
+
+/* Fill `nbytes` bytes at dst_dev with zero (bucket / staging clears:
+ * torch::zeros at src/torch/TorchUtil.cpp:1474, src/comp/ParamStorage.cpp:59-75). */
+int rg_fill_zero(void* dst_dev, int64_t nbytes, int device, void* stream);
+
+/* Results of the last rg_fused_step / rg_unscale_pack / rg_grad_norm on this plan. */
+int rg_result_device_ptr(const rg_plan* plan, const rg_step_result** out_dev);
+int rg_tensor_norms_device_ptr(const rg_plan* plan, const float** out_dev);
+/* These two wait for the stream, then copy to host memory. */
+int rg_read_result(rg_plan* plan, rg_step_result* out_host, void* stream);
+int rg_read_tensor_norms(rg_plan* plan, float* out_host, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RANNCGRAD_H */

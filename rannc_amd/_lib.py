@@ -1,0 +1,206 @@
+"""ctypes binding of libranncgrad.so (the C ABI declared in ``include/ranncgrad.h``).
+
+The library is the only compute path: there is no CPU or PyTorch fallback.  If the
+shared object is missing every import of this module raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import List, Optional, Sequence
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libranncgrad.so")
+
+RG_OK, RG_EINVAL, RG_EALIGN, RG_EHIP, RG_ENOMEM = 0, 1, 2, 3, 4
+RG_F32, RG_F16, RG_BF16 = 0, 1, 2
+RG_STEP_DEFAULT, RG_STEP_WRITE_ON_OVERFLOW, RG_STEP_IGNORE_OVERFLOW = 0, 1, 2
+
+DTYPE_CODES = {"f32": RG_F32, "f16": RG_F16, "bf16": RG_BF16}
+
+
+class StepResult(C.Structure):
+    _fields_ = [("norm", C.c_double), ("coef", C.c_float), ("overflow", C.c_int32),
+                ("clipped", C.c_int32), ("skipped", C.c_int32)]
+
+
+# name -> (restype, argtypes); the complete export list of include/ranncgrad.h
+_vp, _i, _i64, _f = C.c_void_p, C.c_int, C.c_int64, C.c_float
+_pi64, _pi, _pvp = C.POINTER(C.c_int64), C.POINTER(C.c_int), C.POINTER(C.c_void_p)
+SIGNATURES = {
+    "rg_last_error": (C.c_char_p, []),
+    "rg_version": (_i, []),
+    "rg_elem_size": (_i, [_i]),
+    "rg_aligned_numel": (_i64, [_i64, _i, _i]),
+    "rg_segment_layout": (_i, [_i64, _i, _i, _pi64, _pi64, _pi64, _pi64]),
+    "rg_bucket_layout": (_i, [_i, _pi64, _pi, _pi64, _pi64]),
+    "rg_plan_create": (_i, [C.POINTER(_vp), _i, _i, _pvp, _pvp, _pi64, _pi, _pi, _i64]),
+    "rg_plan_update_pointers": (_i, [_vp, _pvp, _pvp, _vp]),
+    "rg_plan_destroy": (_i, [_vp]),
+    "rg_plan_num_tensors": (_i, [_vp]),
+    "rg_plan_num_chunks": (_i64, [_vp]),
+    "rg_plan_chunk_elems": (_i64, [_vp]),
+    "rg_plan_total_numel": (_i64, [_vp]),
+    "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
+    "rg_unscale_pack": (_i, [_vp, _f, _vp]),
+    "rg_grad_norm": (_i, [_vp, _vp]),
+    "rg_scale_cast": (_i, [_vp, _f, _vp]),
+    "rg_zero": (_i, [_vp, _vp]),
+    "rg_fill_zero": (_i, [_vp, _i64, _i, _vp]),
+    "rg_result_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
+    "rg_tensor_norms_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
+    "rg_read_result": (_i, [_vp, C.POINTER(StepResult), _vp]),
+    "rg_read_tensor_norms": (_i, [_vp, C.POINTER(C.c_float), _vp]),
+}
+
+
+class RanncGradError(RuntimeError):
+    pass
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m rannc_amd.build` "
+            "(there is no fallback path)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def check(rc: int) -> None:
+    """Status -> exception, mirroring the reference's pybind translation
+    (std::invalid_argument -> ValueError, std::runtime_error -> RuntimeError)."""
+    if rc == RG_OK:
+        return
+    msg = (lib.rg_last_error() or b"").decode("utf-8", "replace")
+    if rc in (RG_EINVAL, RG_EALIGN):
+        raise ValueError(msg)
+    if rc == RG_ENOMEM:
+        raise MemoryError(msg)
+    raise RanncGradError(msg)
+
+
+# ------------------------------------------------------------------------- layout
+
+def aligned_numel(numel: int, elem_size: int, split_num: int) -> int:
+    r = lib.rg_aligned_numel(numel, elem_size, split_num)
+    if r < 0:
+        check(RG_EINVAL)
+    return int(r)
+
+
+def segment_layout(numel: int, elem_size: int, nranks: int):
+    """-> (aligned_size, segment_size, offsets, src_sizes)."""
+    if nranks < 1:
+        raise ValueError("nranks must be >= 1")
+    aligned, seg = C.c_int64(), C.c_int64()
+    offs, srcs = (C.c_int64 * nranks)(), (C.c_int64 * nranks)()
+    check(lib.rg_segment_layout(numel, elem_size, nranks, C.byref(aligned), C.byref(seg), offs, srcs))
+    return int(aligned.value), int(seg.value), list(offs), list(srcs)
+
+
+def bucket_layout(numels: Sequence[int], dtype_codes: Sequence[int]):
+    """-> (offsets, [len_f32, len_f16, len_bf16])."""
+    n = len(numels)
+    a_n = (C.c_int64 * max(n, 1))(*numels)
+    a_d = (C.c_int * max(n, 1))(*dtype_codes)
+    offs = (C.c_int64 * max(n, 1))()
+    lens = (C.c_int64 * 3)()
+    check(lib.rg_bucket_layout(n, a_n, a_d, offs, lens))
+    return list(offs)[:n], list(lens)
+
+
+# ------------------------------------------------------------------------- plans
+
+class Plan:
+    """Owner of one ``rg_plan``.  Pointers are plain integers (``tensor.data_ptr()``)."""
+
+    def __init__(self, device: int, src_ptrs: Sequence[Optional[int]], dst_ptrs: Sequence[Optional[int]],
+                 numels: Sequence[int], src_dtypes: Sequence[int], dst_dtypes: Sequence[int],
+                 chunk_elems: int = 0):
+        n = len(numels)
+        if not (len(src_ptrs) == len(dst_ptrs) == len(src_dtypes) == len(dst_dtypes) == n):
+            raise ValueError("plan arrays differ in length")
+        self._handle = _vp()
+        self.n = n
+        self.device = device
+        m = max(n, 1)
+        check(lib.rg_plan_create(
+            C.byref(self._handle), device, n,
+            (_vp * m)(*[p or None for p in src_ptrs]), (_vp * m)(*[p or None for p in dst_ptrs]),
+            (C.c_int64 * m)(*numels), (C.c_int * m)(*src_dtypes), (C.c_int * m)(*dst_dtypes),
+            chunk_elems))
+
+    # -- bookkeeping
+    def close(self) -> None:
+        if getattr(self, "_handle", None) is not None and self._handle.value:
+            lib.rg_plan_destroy(self._handle)
+            self._handle = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def num_chunks(self) -> int:
+        return int(lib.rg_plan_num_chunks(self._handle))
+
+    @property
+    def chunk_elems(self) -> int:
+        return int(lib.rg_plan_chunk_elems(self._handle))
+
+    @property
+    def total_numel(self) -> int:
+        return int(lib.rg_plan_total_numel(self._handle))
+
+    def update_pointers(self, src_ptrs: Optional[Sequence[Optional[int]]],
+                        dst_ptrs: Optional[Sequence[Optional[int]]], stream: int = 0) -> None:
+        m = max(self.n, 1)
+        a_s = (_vp * m)(*[p or None for p in src_ptrs]) if src_ptrs is not None else None
+        a_d = (_vp * m)(*[p or None for p in dst_ptrs]) if dst_ptrs is not None else None
+        check(lib.rg_plan_update_pointers(self._handle, a_s, a_d, _vp(stream)))
+
+    # -- operations (all stream ordered)
+    def fused_step(self, inv_scale: float, max_norm: float, flags: int = RG_STEP_DEFAULT, stream: int = 0) -> None:
+        check(lib.rg_fused_step(self._handle, inv_scale, max_norm, flags, _vp(stream)))
+
+    def unscale_pack(self, inv_scale: float, stream: int = 0) -> None:
+        check(lib.rg_unscale_pack(self._handle, inv_scale, _vp(stream)))
+
+    def grad_norm(self, stream: int = 0) -> None:
+        check(lib.rg_grad_norm(self._handle, _vp(stream)))
+
+    def scale_cast(self, scale: float = 1.0, stream: int = 0) -> None:
+        check(lib.rg_scale_cast(self._handle, scale, _vp(stream)))
+
+    def zero(self, stream: int = 0) -> None:
+        check(lib.rg_zero(self._handle, _vp(stream)))
+
+    # -- results (these wait for the stream)
+    def read_result(self, stream: int = 0) -> StepResult:
+        out = StepResult()
+        check(lib.rg_read_result(self._handle, C.byref(out), _vp(stream)))
+        return out
+
+    def read_tensor_norms(self, stream: int = 0) -> List[float]:
+        buf = (C.c_float * max(self.n, 1))()
+        check(lib.rg_read_tensor_norms(self._handle, buf, _vp(stream)))
+        return list(buf)[: self.n]
+
+    def result_device_ptr(self) -> int:
+        out = _vp()
+        check(lib.rg_result_device_ptr(self._handle, C.byref(out)))
+        return int(out.value)
+
+
+def fill_zero(ptr: int, nbytes: int, device: int, stream: int = 0) -> None:
+    check(lib.rg_fill_zero(_vp(ptr), nbytes, device, _vp(stream)))

@@ -1,0 +1,46 @@
+"""Build libranncgrad.so (the HIP kernel library) in-tree for gfx950.
+
+Run as ``python -m rannc_amd.build``; ``__graft_entry__.build()`` calls :func:`build`.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+LIB_NAME = "libranncgrad.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+SOURCES = ["rg_kernels.hip", "rg_api.hip"]
+
+# -ffp-contract=off: the unscale and clip multiplies must stay two roundings.
+# The packed-fp32 feature is switched off for every HIP translation unit of this project.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+    "-ffp-contract=off", "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+def build(verbose: bool = True) -> str:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    srcs = [os.path.join(HERE, "csrc", s) for s in SOURCES]
+    cmd = [hipcc, *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "csrc"),
+           "-o", LIB_PATH + ".tmp", *srcs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if verbose and out.strip():
+        print(out, flush=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{proc.stdout}")
+    os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,527 @@
+// Host side of libranncgrad: layout arithmetic, plans (descriptor + chunk tables resident on
+// the device) and the extern "C" entry points declared in include/ranncgrad.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <new>
+#include <vector>
+
+#include "rg_internal.h"
+
+namespace rg {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+static int hip_fail(hipError_t e, const char* what) {
+  set_error("%s: %s", what, hipGetErrorString(e));
+  return RG_EHIP;
+}
+
+#define RG_HIP(call)                                  \
+  do {                                                \
+    hipError_t e_ = (call);                           \
+    if (e_ != hipSuccess) return hip_fail(e_, #call); \
+  } while (0)
+
+static inline int elem_size(int dtype) {
+  switch (dtype) {
+    case RG_F32: return 4;
+    case RG_F16: return 2;
+    case RG_BF16: return 2;
+    default: return -1;
+  }
+}
+
+static inline int64_t round_up(int64_t x, int64_t q) { return (x + q - 1) / q * q; }
+
+// Makes the plan's device current for the scope of a call and restores the caller's.
+class DeviceGuard {
+ public:
+  explicit DeviceGuard(int device) : prev_(-1), changed_(false) {
+    if (hipGetDevice(&prev_) == hipSuccess && prev_ != device) changed_ = (hipSetDevice(device) == hipSuccess);
+  }
+  ~DeviceGuard() {
+    if (changed_) (void)hipSetDevice(prev_);
+  }
+
+ private:
+  int prev_;
+  bool changed_;
+};
+
+}  // namespace rg
+
+using namespace rg;
+
+struct rg_plan {
+  int device = 0;
+  int n_tensors = 0;
+  int64_t total_numel = 0;
+  int64_t chunk_elems = 0;
+  int64_t n_chunks = 0;
+  std::vector<TensorDesc> host_tensors;
+
+  // one device allocation, carved up
+  char* dev_base = nullptr;
+  size_t dev_bytes = 0;
+  TensorDesc* d_tensors = nullptr;
+  int32_t* d_chunk_tensor = nullptr;
+  int32_t* d_chunk_index = nullptr;
+  int64_t* d_tensor_chunk_begin = nullptr;
+  double* d_chunk_sumsq = nullptr;
+  int32_t* d_chunk_bad = nullptr;
+  float* d_tensor_norm = nullptr;
+  double* d_tensor_sq = nullptr;
+  int32_t* d_tensor_bad = nullptr;
+  unsigned int* d_ticket = nullptr;
+  StepResult* d_result = nullptr;
+
+  // pinned host memory: two descriptor staging buffers (pointer updates stay stream
+  // ordered without a host wait in the common case) and a read-back area
+  char* pinned = nullptr;
+  TensorDesc* stage[2] = {nullptr, nullptr};
+  hipEvent_t stage_done[2] = {nullptr, nullptr};
+  bool stage_used[2] = {false, false};
+  int next_stage = 0;
+  StepResult* h_result = nullptr;
+  float* h_norms = nullptr;
+};
+
+static int check_pointer(const void* p, int esz, const char* which, int i) {
+  if (p != nullptr && (reinterpret_cast<uintptr_t>(p) % (uintptr_t)esz) != 0) {
+    set_error("%s[%d] = %p is not aligned to its %d-byte element", which, i, p, esz);
+    return RG_EALIGN;
+  }
+  return RG_OK;
+}
+
+// ---------------------------------------------------------------------------- misc
+
+RG_API const char* rg_last_error(void) { return g_error; }
+RG_API int rg_version(void) { return RG_VERSION; }
+RG_API int rg_elem_size(int dtype) { return elem_size(dtype); }
+
+// ---------------------------------------------------------------------------- layout
+
+RG_API int64_t rg_aligned_numel(int64_t numel, int esz, int split_num) {
+  if (numel < 0 || split_num < 1 || esz < 1 || 16 % esz != 0) {
+    set_error("rg_aligned_numel: bad arguments (numel=%lld elem_size=%d split=%d)", (long long)numel, esz, split_num);
+    return -1;
+  }
+  const int64_t unit = (int64_t)(16 / esz) * split_num;
+  return round_up(numel, unit);
+}
+
+RG_API int rg_segment_layout(int64_t numel, int esz, int nranks, int64_t* aligned_size, int64_t* segment_size,
+                             int64_t* offsets, int64_t* src_sizes) {
+  const int64_t aligned = rg_aligned_numel(numel, esz, nranks);
+  if (aligned < 0 || offsets == nullptr || src_sizes == nullptr) {
+    if (aligned >= 0) set_error("rg_segment_layout: null output array");
+    return RG_EINVAL;
+  }
+  const int64_t seg = aligned / nranks;
+  int64_t off = 0;
+  for (int i = 0; i < nranks; ++i) {
+    offsets[i] = off;
+    const int64_t rest = numel - off;
+    src_sizes[i] = rest < seg ? rest : seg;
+    off += src_sizes[i];
+  }
+  if (aligned_size) *aligned_size = aligned;
+  if (segment_size) *segment_size = seg;
+  return RG_OK;
+}
+
+RG_API int rg_bucket_layout(int n, const int64_t* numels, const int* dtypes, int64_t* offsets,
+                            int64_t bucket_lengths[3]) {
+  if (n < 0 || (n > 0 && (numels == nullptr || dtypes == nullptr || offsets == nullptr)) || bucket_lengths == nullptr) {
+    set_error("rg_bucket_layout: bad arguments");
+    return RG_EINVAL;
+  }
+  int64_t running[3] = {0, 0, 0};
+  for (int i = 0; i < n; ++i) {
+    if (elem_size(dtypes[i]) < 0 || numels[i] < 0) {
+      set_error("rg_bucket_layout: tensor %d has dtype %d / numel %lld", i, dtypes[i], (long long)numels[i]);
+      return RG_EINVAL;
+    }
+    offsets[i] = running[dtypes[i]];
+    running[dtypes[i]] += numels[i];
+  }
+  for (int k = 0; k < 3; ++k) bucket_lengths[k] = running[k];
+  return RG_OK;
+}
+
+// ---------------------------------------------------------------------------- plans
+
+static int64_t default_chunk_elems(int64_t total) {
+  // Enough chunks to keep 256 compute units busy several times over, but never so small
+  // that the per-chunk table lookup and reduction epilogue show.
+  const int64_t kMax = 16384, kMin = kChunkQuantum, kTargetChunks = 4096;
+  int64_t c = round_up(total / kTargetChunks + 1, kChunkQuantum);
+  if (c < kMin) c = kMin;
+  if (c > kMax) c = kMax;
+  return c;
+}
+
+RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* src, void* const* dst,
+                          const int64_t* numel, const int* src_dtype, const int* dst_dtype, int64_t chunk_elems) {
+  if (out == nullptr || n < 0 || (n > 0 && (numel == nullptr || src_dtype == nullptr || dst_dtype == nullptr))) {
+    set_error("rg_plan_create: bad arguments");
+    return RG_EINVAL;
+  }
+  *out = nullptr;
+  if (chunk_elems < 0 || chunk_elems % kChunkQuantum != 0) {
+    set_error("rg_plan_create: chunk_elems %lld is not a multiple of %lld", (long long)chunk_elems, (long long)kChunkQuantum);
+    return RG_EINVAL;
+  }
+  rg_plan* p = new (std::nothrow) rg_plan();
+  if (p == nullptr) return RG_ENOMEM;
+  p->device = device;
+  p->n_tensors = n;
+  p->host_tensors.resize((size_t)n);
+  int64_t total = 0;
+  for (int i = 0; i < n; ++i) {
+    const int ss = elem_size(src_dtype[i]), ds = elem_size(dst_dtype[i]);
+    if (ss < 0 || ds < 0 || numel[i] < 0) {
+      set_error("rg_plan_create: tensor %d has dtypes %d->%d / numel %lld", i, src_dtype[i], dst_dtype[i], (long long)numel[i]);
+      delete p;
+      return RG_EINVAL;
+    }
+    TensorDesc& t = p->host_tensors[(size_t)i];
+    t.src = src ? src[i] : nullptr;
+    t.dst = dst ? dst[i] : nullptr;
+    t.numel = numel[i];
+    t.src_dtype = src_dtype[i];
+    t.dst_dtype = dst_dtype[i];
+    int rc = check_pointer(t.src, ss, "src", i);
+    if (rc == RG_OK) rc = check_pointer(t.dst, ds, "dst", i);
+    if (rc != RG_OK) {
+      delete p;
+      return rc;
+    }
+    total += numel[i];
+  }
+  p->total_numel = total;
+  p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total);
+
+  std::vector<int64_t> begin((size_t)n + 1, 0);
+  for (int i = 0; i < n; ++i) begin[(size_t)i + 1] = begin[(size_t)i] + (numel[i] + p->chunk_elems - 1) / p->chunk_elems;
+  p->n_chunks = begin[(size_t)n];
+  if (p->n_chunks > 0x7fffffffLL) {
+    set_error("rg_plan_create: %lld chunks exceed the grid limit; raise chunk_elems", (long long)p->n_chunks);
+    delete p;
+    return RG_EINVAL;
+  }
+  std::vector<int32_t> chunk_tensor((size_t)p->n_chunks), chunk_index((size_t)p->n_chunks);
+  for (int i = 0; i < n; ++i)
+    for (int64_t c = begin[(size_t)i]; c < begin[(size_t)i + 1]; ++c) {
+      chunk_tensor[(size_t)c] = i;
+      chunk_index[(size_t)c] = (int32_t)(c - begin[(size_t)i]);
+    }
+
+  // carve one device allocation
+  size_t off = 0;
+  auto carve = [&off](size_t bytes) {
+    const size_t at = off;
+    off += (bytes + 255) / 256 * 256;
+    return at;
+  };
+  const size_t nt = (size_t)(n > 0 ? n : 1), nc = (size_t)(p->n_chunks > 0 ? p->n_chunks : 1);
+  const size_t o_tensors = carve(nt * sizeof(TensorDesc));
+  const size_t o_ctensor = carve(nc * sizeof(int32_t));
+  const size_t o_cindex = carve(nc * sizeof(int32_t));
+  const size_t o_begin = carve((nt + 1) * sizeof(int64_t));
+  const size_t o_sumsq = carve(nc * sizeof(double));
+  const size_t o_bad = carve(nc * sizeof(int32_t));
+  const size_t o_tnorm = carve(nt * sizeof(float));
+  const size_t o_tsq = carve(nt * sizeof(double));
+  const size_t o_tbad = carve(nt * sizeof(int32_t));
+  const size_t o_ticket = carve(sizeof(unsigned int));
+  const size_t o_result = carve(sizeof(StepResult));
+  p->dev_bytes = off;
+
+  DeviceGuard guard(device);
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&p->dev_base), p->dev_bytes);
+  if (e != hipSuccess) {
+    delete p;
+    return hip_fail(e, "hipMalloc(plan tables)");
+  }
+  char* b = p->dev_base;
+  p->d_tensors = reinterpret_cast<TensorDesc*>(b + o_tensors);
+  p->d_chunk_tensor = reinterpret_cast<int32_t*>(b + o_ctensor);
+  p->d_chunk_index = reinterpret_cast<int32_t*>(b + o_cindex);
+  p->d_tensor_chunk_begin = reinterpret_cast<int64_t*>(b + o_begin);
+  p->d_chunk_sumsq = reinterpret_cast<double*>(b + o_sumsq);
+  p->d_chunk_bad = reinterpret_cast<int32_t*>(b + o_bad);
+  p->d_tensor_norm = reinterpret_cast<float*>(b + o_tnorm);
+  p->d_tensor_sq = reinterpret_cast<double*>(b + o_tsq);
+  p->d_tensor_bad = reinterpret_cast<int32_t*>(b + o_tbad);
+  p->d_ticket = reinterpret_cast<unsigned int*>(b + o_ticket);
+  p->d_result = reinterpret_cast<StepResult*>(b + o_result);
+
+  const size_t stage_bytes = (nt * sizeof(TensorDesc) + 255) / 256 * 256;
+  const size_t norms_bytes = (nt * sizeof(float) + 255) / 256 * 256;
+  e = hipHostMalloc(reinterpret_cast<void**>(&p->pinned), 2 * stage_bytes + 256 + norms_bytes, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    (void)hipFree(p->dev_base);
+    delete p;
+    return hip_fail(e, "hipHostMalloc(plan staging)");
+  }
+  p->stage[0] = reinterpret_cast<TensorDesc*>(p->pinned);
+  p->stage[1] = reinterpret_cast<TensorDesc*>(p->pinned + stage_bytes);
+  p->h_result = reinterpret_cast<StepResult*>(p->pinned + 2 * stage_bytes);
+  p->h_norms = reinterpret_cast<float*>(p->pinned + 2 * stage_bytes + 256);
+
+  bool ok = hipMemset(p->dev_base, 0, p->dev_bytes) == hipSuccess;
+  if (ok && n > 0) ok = hipMemcpy(p->d_tensors, p->host_tensors.data(), (size_t)n * sizeof(TensorDesc), hipMemcpyHostToDevice) == hipSuccess;
+  if (ok) ok = hipMemcpy(p->d_tensor_chunk_begin, begin.data(), begin.size() * sizeof(int64_t), hipMemcpyHostToDevice) == hipSuccess;
+  if (ok && p->n_chunks > 0) {
+    ok = hipMemcpy(p->d_chunk_tensor, chunk_tensor.data(), chunk_tensor.size() * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess &&
+         hipMemcpy(p->d_chunk_index, chunk_index.data(), chunk_index.size() * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess;
+  }
+  for (int k = 0; ok && k < 2; ++k) ok = hipEventCreateWithFlags(&p->stage_done[k], hipEventDisableTiming) == hipSuccess;
+  if (!ok) {
+    const hipError_t last = hipGetLastError();
+    rg_plan_destroy(p);
+    return hip_fail(last, "rg_plan_create: uploading the tables");
+  }
+  *out = p;
+  return RG_OK;
+}
+
+RG_API int rg_plan_destroy(rg_plan* p) {
+  if (p == nullptr) return RG_OK;
+  DeviceGuard guard(p->device);
+  (void)hipDeviceSynchronize();
+  for (int k = 0; k < 2; ++k)
+    if (p->stage_done[k]) (void)hipEventDestroy(p->stage_done[k]);
+  if (p->pinned) (void)hipHostFree(p->pinned);
+  if (p->dev_base) (void)hipFree(p->dev_base);
+  delete p;
+  return RG_OK;
+}
+
+RG_API int rg_plan_update_pointers(rg_plan* p, const void* const* src, void* const* dst, void* stream) {
+  if (p == nullptr) {
+    set_error("rg_plan_update_pointers: null plan");
+    return RG_EINVAL;
+  }
+  const int n = p->n_tensors;
+  for (int i = 0; i < n; ++i) {
+    const TensorDesc& t = p->host_tensors[(size_t)i];
+    int rc = RG_OK;
+    if (src) rc = check_pointer(src[i], elem_size(t.src_dtype), "src", i);
+    if (rc == RG_OK && dst) rc = check_pointer(dst[i], elem_size(t.dst_dtype), "dst", i);
+    if (rc != RG_OK) return rc;
+  }
+  for (int i = 0; i < n; ++i) {
+    if (src) p->host_tensors[(size_t)i].src = src[i];
+    if (dst) p->host_tensors[(size_t)i].dst = dst[i];
+  }
+  if (n == 0) return RG_OK;
+  DeviceGuard guard(p->device);
+  const int k = p->next_stage;
+  p->next_stage ^= 1;
+  if (p->stage_used[k]) RG_HIP(hipEventSynchronize(p->stage_done[k]));
+  memcpy(p->stage[k], p->host_tensors.data(), (size_t)n * sizeof(TensorDesc));
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  RG_HIP(hipMemcpyAsync(p->d_tensors, p->stage[k], (size_t)n * sizeof(TensorDesc), hipMemcpyHostToDevice, s));
+  RG_HIP(hipEventRecord(p->stage_done[k], s));
+  p->stage_used[k] = true;
+  return RG_OK;
+}
+
+RG_API int rg_plan_num_tensors(const rg_plan* p) { return p ? p->n_tensors : -1; }
+RG_API int64_t rg_plan_num_chunks(const rg_plan* p) { return p ? p->n_chunks : -1; }
+RG_API int64_t rg_plan_chunk_elems(const rg_plan* p) { return p ? p->chunk_elems : -1; }
+RG_API int64_t rg_plan_total_numel(const rg_plan* p) { return p ? p->total_numel : -1; }
+
+// ---------------------------------------------------------------------------- operations
+
+static PassArgs pass_args(const rg_plan* p, float scale) {
+  PassArgs a;
+  a.tensors = p->d_tensors;
+  a.chunk_tensor = p->d_chunk_tensor;
+  a.chunk_index = p->d_chunk_index;
+  a.chunk_sumsq = p->d_chunk_sumsq;
+  a.chunk_bad = p->d_chunk_bad;
+  a.result = nullptr;
+  a.chunk_elems = p->chunk_elems;
+  a.n_chunks = p->n_chunks;
+  a.scale = scale;
+  a.write_on_overflow = 0;
+  a.reverse = 0;
+  a.zero_fill = 0;
+  a.norm_of_source = 0;
+  return a;
+}
+
+static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_overflow) {
+  FinalizeArgs f;
+  f.tensor_chunk_begin = p->d_tensor_chunk_begin;
+  f.chunk_sumsq = p->d_chunk_sumsq;
+  f.chunk_bad = p->d_chunk_bad;
+  f.tensor_norm = p->d_tensor_norm;
+  f.tensor_sq = p->d_tensor_sq;
+  f.tensor_bad = p->d_tensor_bad;
+  f.ticket = p->d_ticket;
+  f.result = p->d_result;
+  f.n_tensors = p->n_tensors;
+  f.max_norm = max_norm;
+  f.ignore_overflow = ignore_overflow;
+  return f;
+}
+
+// Which pointers an operation dereferences.
+enum { kNeedSrc = 1, kNeedDst = 2 };
+
+static int check_plan(const rg_plan* p, int need, const char* op) {
+  if (p == nullptr) {
+    set_error("%s: null plan", op);
+    return RG_EINVAL;
+  }
+  for (int i = 0; i < p->n_tensors; ++i) {
+    const TensorDesc& t = p->host_tensors[(size_t)i];
+    if (t.numel == 0) continue;
+    if ((need & kNeedDst) && t.dst == nullptr) {
+      set_error("%s: tensor %d has no destination pointer", op, i);
+      return RG_EINVAL;
+    }
+    if ((need & kNeedDst) && t.dst == t.src && t.src_dtype != t.dst_dtype) {
+      set_error("%s: tensor %d is in place but changes dtype", op, i);
+      return RG_EINVAL;
+    }
+  }
+  return RG_OK;
+}
+
+RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags, void* stream) {
+  const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_fused_step");
+  if (rc != RG_OK) return rc;
+  if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
+    set_error("rg_fused_step: inv_scale must be a non-zero number");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  PassArgs a = pass_args(p, inv_scale);
+  RG_HIP(launch_pass(kModeReduce, a, s));
+  RG_HIP(launch_finalize(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
+  a.result = p->d_result;
+  a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
+  // Walk the chunks backwards: the tail of pass 1 is what the caches still hold.
+  a.reverse = 1;
+  RG_HIP(launch_pass(kModeWrite, a, s));
+  return RG_OK;
+}
+
+RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
+  const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_unscale_pack");
+  if (rc != RG_OK) return rc;
+  if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
+    set_error("rg_unscale_pack: inv_scale must be a non-zero number");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  RG_HIP(launch_pass(kModeReduce | kModeWrite, pass_args(p, inv_scale), s));
+  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
+  return RG_OK;
+}
+
+RG_API int rg_grad_norm(rg_plan* p, void* stream) {
+  const int rc = check_plan(p, kNeedSrc, "rg_grad_norm");
+  if (rc != RG_OK) return rc;
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  PassArgs a = pass_args(p, 1.0f);
+  a.norm_of_source = 1;
+  RG_HIP(launch_pass(kModeReduce, a, s));
+  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 1), s));
+  return RG_OK;
+}
+
+RG_API int rg_scale_cast(rg_plan* p, float scale, void* stream) {
+  const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_scale_cast");
+  if (rc != RG_OK) return rc;
+  DeviceGuard guard(p->device);
+  RG_HIP(launch_pass(kModeWrite, pass_args(p, scale), reinterpret_cast<hipStream_t>(stream)));
+  return RG_OK;
+}
+
+RG_API int rg_zero(rg_plan* p, void* stream) {
+  const int rc = check_plan(p, kNeedDst, "rg_zero");
+  if (rc != RG_OK) return rc;
+  DeviceGuard guard(p->device);
+  PassArgs a = pass_args(p, 1.0f);
+  a.zero_fill = 1;
+  RG_HIP(launch_pass(kModeWrite, a, reinterpret_cast<hipStream_t>(stream)));
+  return RG_OK;
+}
+
+RG_API int rg_fill_zero(void* dst_dev, int64_t nbytes, int device, void* stream) {
+  if (nbytes < 0 || (nbytes > 0 && dst_dev == nullptr)) {
+    set_error("rg_fill_zero: bad arguments");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(device);
+  RG_HIP(launch_fill_zero(dst_dev, nbytes, reinterpret_cast<hipStream_t>(stream)));
+  return RG_OK;
+}
+
+RG_API int rg_result_device_ptr(const rg_plan* p, const rg_step_result** out_dev) {
+  if (p == nullptr || out_dev == nullptr) {
+    set_error("rg_result_device_ptr: null argument");
+    return RG_EINVAL;
+  }
+  *out_dev = reinterpret_cast<const rg_step_result*>(p->d_result);
+  return RG_OK;
+}
+
+RG_API int rg_tensor_norms_device_ptr(const rg_plan* p, const float** out_dev) {
+  if (p == nullptr || out_dev == nullptr) {
+    set_error("rg_tensor_norms_device_ptr: null argument");
+    return RG_EINVAL;
+  }
+  *out_dev = p->d_tensor_norm;
+  return RG_OK;
+}
+
+RG_API int rg_read_result(rg_plan* p, rg_step_result* out_host, void* stream) {
+  if (p == nullptr || out_host == nullptr) {
+    set_error("rg_read_result: null argument");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  RG_HIP(hipMemcpyAsync(p->h_result, p->d_result, sizeof(StepResult), hipMemcpyDeviceToHost, s));
+  RG_HIP(hipStreamSynchronize(s));
+  out_host->norm = p->h_result->norm;
+  out_host->coef = p->h_result->coef;
+  out_host->overflow = p->h_result->overflow;
+  out_host->clipped = p->h_result->clipped;
+  out_host->skipped = p->h_result->skipped;
+  return RG_OK;
+}
+
+RG_API int rg_read_tensor_norms(rg_plan* p, float* out_host, void* stream) {
+  if (p == nullptr || (p->n_tensors > 0 && out_host == nullptr)) {
+    set_error("rg_read_tensor_norms: null argument");
+    return RG_EINVAL;
+  }
+  if (p->n_tensors == 0) return RG_OK;
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  RG_HIP(hipMemcpyAsync(p->h_norms, p->d_tensor_norm, (size_t)p->n_tensors * sizeof(float), hipMemcpyDeviceToHost, s));
+  RG_HIP(hipStreamSynchronize(s));
+  memcpy(out_host, p->h_norms, (size_t)p->n_tensors * sizeof(float));
+  return RG_OK;
+}
