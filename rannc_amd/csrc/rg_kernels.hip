@@ -74,7 +74,8 @@ template <> __device__ __forceinline__ void unpack<RG_F32>(const Raw<RG_F32>& r,
 template <> __device__ __forceinline__ void unpack<RG_F16>(const Raw<RG_F16>& r, float (&f)[8]) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const f16x2 h = __builtin_bit_cast(f16x2, r.a[j]);
+    const unsigned int w = r.a[j];  // bit_cast must see a scalar, not a vector-element lvalue
+    const f16x2 h = __builtin_bit_cast(f16x2, w);
     f[2 * j] = (float)h.x;
     f[2 * j + 1] = (float)h.y;
   }

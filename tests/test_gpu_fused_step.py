@@ -58,7 +58,7 @@ def _check_against_oracle(grads_cpu, dst_name, inv_scale, max_norm, res, tnorms,
         assert math.isclose(a, b, rel_tol=REL, abs_tol=1e-30), (i, a, b)
     assert res.clipped == (1 if want.coef is not None else 0)
     # unscaled bucket from the oracle, then the GPU's own coefficient applied on the CPU
-    unscaled = oracle.fused_step(grads_cpu, [dst_name] * n, inv_scale, 0.0).buckets.get(dst_name)
+    unscaled = oracle.fused_step(grads_cpu, [dst_name] * n, inv_scale, math.inf).buckets.get(dst_name)
     if unscaled is None:
         unscaled = torch.zeros(0, dtype=TORCH_DTYPE[dst_name])
     if want.coef is not None:
