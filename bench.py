@@ -1,0 +1,187 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused unscale + overflow-check + norm + clip + pack step on one MI355X.
+
+A "step" is one pass of the fused step over one batch of synthetic gradients that are already
+resident in HBM: pass 1 reads the gradients (flag + per-tensor sums of squares), a small
+kernel derives the global norm and the clip coefficient on the device, pass 2 re-reads the
+gradients and writes the unscaled, clipped values into the packed fp32 bucket.
+
+Prints ONE JSON line.  `value` is algorithmic GB/s over the whole step: (2*s + d) * N bytes
+(s, d = source / destination bytes per element) divided by the measured time per step.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import platform
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+
+# HBM traffic per launch of the dominant kernel (the write pass), from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of this same command; see profiles/.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2_bert_large")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--chunk-elems", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget for the CPU baseline leg")
+    return ap.parse_args()
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return platform.processor() or "unknown"
+
+
+def cpu_baseline(cfg, seed: int, budget_s: float):
+    """The reference's op sequence on the host cores (oracle.reference_step_cpu), on a bounded
+    sample of the same workload: the same tensor list with dim 0 of every tensor scaled so
+    that one CPU step fits the budget several times."""
+    import torch
+    from oracle import gradpath as oracle
+    from rannc_amd.workloads import make_grads
+
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    frac = 1.0
+    # ~0.3 GB/s per thread is a safe lower bound for the per-tensor op chain
+    est = cfg.total_numel * 8 / (0.3e9 * threads)
+    if est > budget_s / 4:
+        frac = max(0.02, (budget_s / 4) / est)
+    grads, _ = make_grads(cfg, seed, device="cpu", scale_numel=frac)
+    n = sum(g.numel() for g in grads)
+    ddt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[cfg.bucket_dtype]
+    bucket = torch.zeros(n, dtype=ddt)
+    views, off = [], 0
+    for g in grads:
+        views.append(bucket.narrow(0, off, g.numel()).view(g.shape))
+        off += g.numel()
+    s, d = grads[0].element_size(), bucket.element_size()
+    best = float("inf")
+    t_start = time.perf_counter()
+    reps = 0
+    while reps < 5 and (reps < 2 or time.perf_counter() - t_start < budget_s):
+        t0 = time.perf_counter()
+        ovf, norm, coef = oracle.reference_step_cpu(grads, views, cfg.inv_scale, cfg.max_norm)
+        dt = time.perf_counter() - t0
+        if reps > 0 or dt > budget_s / 2:
+            best = min(best, dt)
+        reps += 1
+    nbytes = ((2 * s + d) if coef is not None else (s + d)) * n
+    return {
+        "value": round(nbytes / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"{cfg.key}: same {len(grads)}-tensor list, {n} of {cfg.total_numel} elements "
+                  f"(dim-0 fraction {frac:.3f}), best of {max(1, reps - 1)} steps of {best * 1e3:.1f} ms, "
+                  f"torch {torch.__version__} CPU ops, {cpu_model()}",
+        "elements_per_s": round(n / best, 1),
+    }
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
+              "the path has no collectives and shards by running the same kernels per rank",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from rannc_amd.multi_tensor import TensorPlan
+    from rannc_amd.workloads import make_grads, step_config
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    cfg = step_config(args.workload)
+    grads, _ = make_grads(cfg, args.seed, device=str(dev))
+    n = sum(g.numel() for g in grads)
+    ddt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[cfg.bucket_dtype]
+    bucket = torch.zeros(n, dtype=ddt, device=dev)
+    dsts, off = [], 0
+    for g in grads:
+        dsts.append(bucket.narrow(0, off, g.numel()))
+        off += g.numel()
+    s, d = grads[0].element_size(), bucket.element_size()
+
+    plan = TensorPlan(grads, dsts, chunk_elems=args.chunk_elems)
+    for _ in range(args.warmup):
+        plan.fused_step(cfg.inv_scale, cfg.max_norm)
+    torch.cuda.synchronize()
+    plan.plan.enable_timing(args.steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.fused_step(cfg.inv_scale, cfg.max_norm)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    res = plan.result()
+    per_kernel = [plan.plan.read_timing(i) for i in range(args.steps)]
+    plan.plan.enable_timing(0)
+
+    step_s = elapsed / args.steps
+    clipped = bool(res.clipped)
+    step_bytes = ((2 * s + d) if clipped else (s + d)) * n
+    value = step_bytes / step_s / 1e9
+
+    # dominant kernel: the write pass (re-read s*N, write d*N)
+    write_ms = sum(k[2] for k in per_kernel) / len(per_kernel)
+    reduce_ms = sum(k[0] for k in per_kernel) / len(per_kernel)
+    final_ms = sum(k[1] for k in per_kernel) / len(per_kernel)
+    write_bytes = (s + d) * n
+    achieved = write_bytes / (write_ms * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm", "kernel": "pass_kernel<write>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.key),
+        "algorithmic_bytes_per_launch": write_bytes, "avg_launch_ms": round(write_ms, 4),
+        "other_kernels": {
+            "pass_kernel<reduce>": {"avg_launch_ms": round(reduce_ms, 4), "algorithmic_bytes_per_launch": s * n,
+                                    "achieved": round(s * n / (reduce_ms * 1e-3) / 1e9, 1)},
+            "finalize_kernel": {"avg_launch_ms": round(final_ms, 4)},
+        },
+    }
+
+    out = {
+        "metric": "achieved HBM GB/s (% of roofline) for fused unscale+norm+clip+pack per step",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": f"{cfg.grad_dtype}->{cfg.bucket_dtype} (fp32 arithmetic)",
+        "data": "synthetic",
+        "config": {"workload": cfg.key, "description": cfg.description, "tensors": len(grads), "elements": n,
+                   "src_bytes_per_elem": s, "dst_bytes_per_elem": d,
+                   "algorithmic_bytes_per_step": step_bytes, "clipped": clipped, "overflow": int(res.overflow),
+                   "norm": res.norm, "coef": res.coef, "seed": args.seed,
+                   "chunk_elems": plan.plan.chunk_elems, "chunks": plan.plan.num_chunks},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "elements_per_s": round(n / step_s, 1),
+        "roofline": roofline,
+    }
+    plan.close()
+    del grads, bucket, dsts
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, args.seed, args.cpu_seconds)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -157,6 +157,17 @@ int rg_tensor_norms_device_ptr(const rg_plan* plan, const float** out_dev);
 int rg_read_result(rg_plan* plan, rg_step_result* out_host, void* stream);
 int rg_read_tensor_norms(rg_plan* plan, float* out_host, void* stream);
 
+/* ---------------------------------------------------------------- per-kernel timing */
+
+/* Optional profiling aid (no counterpart in the reference, which times with its own
+ * TimeCounter around whole calls, src/comp/TimeCounter.cpp:10-27).  With `slots` > 0 every
+ * rg_fused_step records HIP events on its stream around its three kernels into the next
+ * slot of a ring; slots == 0 switches it off.  rg_plan_read_timing waits for that slot and
+ * returns milliseconds: ms[0] reduce pass, ms[1] finalize, ms[2] write pass, ms[3] whole step.
+ * slot counts fused steps since timing was enabled, modulo `slots`. */
+int rg_plan_enable_timing(rg_plan* plan, int slots);
+int rg_plan_read_timing(rg_plan* plan, int slot, float ms[4]);
+
 #ifdef __cplusplus
 }
 #endif

@@ -382,3 +382,37 @@ def patched_update_scale(state: LossScalerState, had_overflow_local: bool,
         state.unskipped = 0
         return True
     return False
+
+
+# --------------------------------------------------------------------------- timed CPU baseline
+
+def reference_step_cpu(model_grads: Sequence[torch.Tensor], master_grad_views: Sequence[torch.Tensor],
+                       inv_scale: float, max_grad_norm: float) -> Tuple[int, float, Optional[float]]:
+    """The reference's per-step work exactly as it issues it on CPU tensors, one ATen op per
+    tensor, writing into preallocated bucket views (used as the timed CPU baseline):
+
+    * unscale + flag per tensor (Apex ``multi_tensor_scale`` semantics; the reference's host
+      loop shape is that of ``src/comp/ParamStorage.cpp:135-178``): ``view.copy_(g)`` casts
+      into the fp32 master-grad view, ``mul_(inv_scale)``, ``isfinite().all()``;
+    * ``norm(2, Float).item()`` per tensor, double sum (``:767-770, 809-818``);
+    * ``mul_(max / (norm + 1e-6))`` per tensor when it exceeds the bound (``:721-745``).
+    Returns (overflow, norm, coef)."""
+    overflow = 0
+    for g, v in zip(model_grads, master_grad_views):
+        v.copy_(g)
+        if inv_scale != 1.0:
+            v.mul_(inv_scale)
+        if g.numel() and not bool(torch.isfinite(v).all()):
+            overflow = 1
+    if overflow:
+        return 1, float("nan"), None
+    norm_sq = 0.0
+    for v in master_grad_views:
+        n = float(v.norm(2, dtype=torch.float32).item())
+        norm_sq += n * n
+    norm = math.sqrt(norm_sq)
+    coef = clip_coefficient(norm, max_grad_norm)
+    if coef is not None:
+        for v in master_grad_views:
+            v.mul_(coef)
+    return 0, norm, coef

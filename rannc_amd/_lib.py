@@ -51,6 +51,8 @@ SIGNATURES = {
     "rg_tensor_norms_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
     "rg_read_result": (_i, [_vp, C.POINTER(StepResult), _vp]),
     "rg_read_tensor_norms": (_i, [_vp, C.POINTER(C.c_float), _vp]),
+    "rg_plan_enable_timing": (_i, [_vp, _i]),
+    "rg_plan_read_timing": (_i, [_vp, _i, C.POINTER(C.c_float)]),
 }
 
 
@@ -195,6 +197,15 @@ class Plan:
         buf = (C.c_float * max(self.n, 1))()
         check(lib.rg_read_tensor_norms(self._handle, buf, _vp(stream)))
         return list(buf)[: self.n]
+
+    def enable_timing(self, slots: int) -> None:
+        check(lib.rg_plan_enable_timing(self._handle, slots))
+
+    def read_timing(self, slot: int) -> List[float]:
+        """[reduce pass, finalize, write pass, whole step] in milliseconds."""
+        ms = (C.c_float * 4)()
+        check(lib.rg_plan_read_timing(self._handle, slot, ms))
+        return list(ms)
 
     def result_device_ptr(self) -> int:
         out = _vp()

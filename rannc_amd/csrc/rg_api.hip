@@ -93,6 +93,11 @@ struct rg_plan {
   int next_stage = 0;
   StepResult* h_result = nullptr;
   float* h_norms = nullptr;
+
+  // optional ring of event quadruples around the kernels of rg_fused_step
+  std::vector<hipEvent_t> timing_events;
+  int timing_slots = 0;
+  int64_t timing_count = 0;
 };
 
 static int check_pointer(const void* p, int esz, const char* which, int i) {
@@ -303,6 +308,7 @@ RG_API int rg_plan_destroy(rg_plan* p) {
   (void)hipDeviceSynchronize();
   for (int k = 0; k < 2; ++k)
     if (p->stage_done[k]) (void)hipEventDestroy(p->stage_done[k]);
+  for (hipEvent_t e : p->timing_events) (void)hipEventDestroy(e);
   if (p->pinned) (void)hipHostFree(p->pinned);
   if (p->dev_base) (void)hipFree(p->dev_base);
   delete p;
@@ -412,14 +418,20 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   }
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  hipEvent_t* ev = nullptr;
+  if (p->timing_slots > 0) ev = &p->timing_events[(size_t)(p->timing_count++ % p->timing_slots) * 4];
   PassArgs a = pass_args(p, inv_scale);
+  if (ev) RG_HIP(hipEventRecord(ev[0], s));
   RG_HIP(launch_pass(kModeReduce, a, s));
+  if (ev) RG_HIP(hipEventRecord(ev[1], s));
   RG_HIP(launch_finalize(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
+  if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
   // Walk the chunks backwards: the tail of pass 1 is what the caches still hold.
   a.reverse = 1;
   RG_HIP(launch_pass(kModeWrite, a, s));
+  if (ev) RG_HIP(hipEventRecord(ev[3], s));
   return RG_OK;
 }
 
@@ -523,5 +535,42 @@ RG_API int rg_read_tensor_norms(rg_plan* p, float* out_host, void* stream) {
   RG_HIP(hipMemcpyAsync(p->h_norms, p->d_tensor_norm, (size_t)p->n_tensors * sizeof(float), hipMemcpyDeviceToHost, s));
   RG_HIP(hipStreamSynchronize(s));
   memcpy(out_host, p->h_norms, (size_t)p->n_tensors * sizeof(float));
+  return RG_OK;
+}
+
+// ---------------------------------------------------------------------------- timing
+
+RG_API int rg_plan_enable_timing(rg_plan* p, int slots) {
+  if (p == nullptr || slots < 0 || slots > 65536) {
+    set_error("rg_plan_enable_timing: bad arguments");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  for (hipEvent_t e : p->timing_events) (void)hipEventDestroy(e);
+  p->timing_events.clear();
+  p->timing_slots = 0;
+  p->timing_count = 0;
+  p->timing_events.reserve((size_t)slots * 4);
+  for (int i = 0; i < slots * 4; ++i) {
+    hipEvent_t e;
+    RG_HIP(hipEventCreate(&e));
+    p->timing_events.push_back(e);
+  }
+  p->timing_slots = slots;
+  return RG_OK;
+}
+
+RG_API int rg_plan_read_timing(rg_plan* p, int slot, float ms[4]) {
+  if (p == nullptr || ms == nullptr || slot < 0 || slot >= p->timing_slots || (int64_t)slot >= p->timing_count) {
+    set_error("rg_plan_read_timing: no timing recorded in slot %d", slot);
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipEvent_t* ev = &p->timing_events[(size_t)slot * 4];
+  RG_HIP(hipEventSynchronize(ev[3]));
+  RG_HIP(hipEventElapsedTime(&ms[0], ev[0], ev[1]));
+  RG_HIP(hipEventElapsedTime(&ms[1], ev[1], ev[2]));
+  RG_HIP(hipEventElapsedTime(&ms[2], ev[2], ev[3]));
+  RG_HIP(hipEventElapsedTime(&ms[3], ev[0], ev[3]));
   return RG_OK;
 }
