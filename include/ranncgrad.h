@@ -91,7 +91,8 @@ int rg_bucket_layout(int n, const int64_t* numels, const int* dtypes, int64_t* o
  * every op is then in place. */
 typedef struct rg_plan rg_plan;
 
-/* chunk_elems: elements per work chunk (multiple of 2048), 0 = choose from the total size. */
+/* chunk_elems: elements per work chunk (multiple of 2048, at most 2^20), 0 = choose from the
+ * total size. */
 int rg_plan_create(rg_plan** out, int device, int n, const void* const* src, void* const* dst,
                    const int64_t* numel, const int* src_dtype, const int* dst_dtype,
                    int64_t chunk_elems);
@@ -102,6 +103,10 @@ int rg_plan_num_tensors(const rg_plan* plan);
 int64_t rg_plan_num_chunks(const rg_plan* plan);
 int64_t rg_plan_chunk_elems(const rg_plan* plan);
 int64_t rg_plan_total_numel(const rg_plan* plan);
+/* Cache policy of the plan's kernels: 1 = nontemporal loads and stores (the data is streamed
+ * once and is far larger than the caches), 0 = plain accesses (the second pass of a small
+ * plan then hits in cache), -1 = decide from the plan's size (the default). */
+int rg_plan_set_streaming(rg_plan* plan, int mode);
 
 /* ---------------------------------------------------------------- per-step operations */
 

@@ -10,7 +10,8 @@ import os
 from typing import List, Optional, Sequence
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libranncgrad.so")
+# RANNC_AMD_LIB points at an alternative build of the same library (tuning experiments).
+LIB_PATH = os.environ.get("RANNC_AMD_LIB") or os.path.join(HERE, "libranncgrad.so")
 
 RG_OK, RG_EINVAL, RG_EALIGN, RG_EHIP, RG_ENOMEM = 0, 1, 2, 3, 4
 RG_F32, RG_F16, RG_BF16 = 0, 1, 2
@@ -41,6 +42,7 @@ SIGNATURES = {
     "rg_plan_num_chunks": (_i64, [_vp]),
     "rg_plan_chunk_elems": (_i64, [_vp]),
     "rg_plan_total_numel": (_i64, [_vp]),
+    "rg_plan_set_streaming": (_i, [_vp, _i]),
     "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
     "rg_unscale_pack": (_i, [_vp, _f, _vp]),
     "rg_grad_norm": (_i, [_vp, _vp]),
@@ -163,6 +165,10 @@ class Plan:
     @property
     def total_numel(self) -> int:
         return int(lib.rg_plan_total_numel(self._handle))
+
+    def set_streaming(self, mode: int) -> None:
+        """1 = nontemporal accesses, 0 = plain, -1 = decide from the plan's size."""
+        check(lib.rg_plan_set_streaming(self._handle, mode))
 
     def update_pointers(self, src_ptrs: Optional[Sequence[Optional[int]]],
                         dst_ptrs: Optional[Sequence[Optional[int]]], stream: int = 0) -> None:

@@ -1,5 +1,5 @@
-// Host side of libranncgrad: layout arithmetic, plans (descriptor + chunk tables resident on
-// the device) and the extern "C" entry points declared in include/ranncgrad.h.
+// Host side of libranncgrad: layout arithmetic, plans (the chunk table resident on the
+// device) and the extern "C" entry points declared in include/ranncgrad.h.
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -65,16 +65,17 @@ struct rg_plan {
   int device = 0;
   int n_tensors = 0;
   int64_t total_numel = 0;
+  int64_t total_bytes = 0;  // source + destination bytes one full pass touches
   int64_t chunk_elems = 0;
   int64_t n_chunks = 0;
+  bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
   std::vector<TensorDesc> host_tensors;
+  std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
 
   // one device allocation, carved up
   char* dev_base = nullptr;
   size_t dev_bytes = 0;
-  TensorDesc* d_tensors = nullptr;
-  int32_t* d_chunk_tensor = nullptr;
-  int32_t* d_chunk_index = nullptr;
+  ChunkRec* d_chunks = nullptr;
   int64_t* d_tensor_chunk_begin = nullptr;
   double* d_chunk_sumsq = nullptr;
   int32_t* d_chunk_bad = nullptr;
@@ -84,10 +85,10 @@ struct rg_plan {
   unsigned int* d_ticket = nullptr;
   StepResult* d_result = nullptr;
 
-  // pinned host memory: two descriptor staging buffers (pointer updates stay stream
+  // pinned host memory: two chunk-table staging buffers (pointer updates stay stream
   // ordered without a host wait in the common case) and a read-back area
   char* pinned = nullptr;
-  TensorDesc* stage[2] = {nullptr, nullptr};
+  ChunkRec* stage[2] = {nullptr, nullptr};
   hipEvent_t stage_done[2] = {nullptr, nullptr};
   bool stage_used[2] = {false, false};
   int next_stage = 0;
@@ -106,6 +107,26 @@ static int check_pointer(const void* p, int esz, const char* which, int i) {
     return RG_EALIGN;
   }
   return RG_OK;
+}
+
+// Writes the chunk records of every tensor into `out` ([n_chunks]).
+static void fill_chunk_records(const rg_plan* p, ChunkRec* out) {
+  for (int i = 0; i < p->n_tensors; ++i) {
+    const TensorDesc& t = p->host_tensors[(size_t)i];
+    const int ss = elem_size(t.src_dtype), ds = elem_size(t.dst_dtype);
+    for (int64_t c = p->chunk_begin[(size_t)i]; c < p->chunk_begin[(size_t)i + 1]; ++c) {
+      const int64_t start = (c - p->chunk_begin[(size_t)i]) * p->chunk_elems;
+      const int64_t rest = t.numel - start;
+      ChunkRec& r = out[c];
+      r.src = t.src ? static_cast<const char*>(t.src) + start * ss : nullptr;
+      r.dst = t.dst ? static_cast<char*>(t.dst) + start * ds : nullptr;
+      r.len = (int32_t)(rest < p->chunk_elems ? rest : p->chunk_elems);
+      r.tensor = i;
+      r.src_dtype = (int16_t)t.src_dtype;
+      r.dst_dtype = (int16_t)t.dst_dtype;
+      r.pad = 0;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------- misc
@@ -168,8 +189,8 @@ RG_API int rg_bucket_layout(int n, const int64_t* numels, const int* dtypes, int
 
 static int64_t default_chunk_elems(int64_t total) {
   // Enough chunks to keep 256 compute units busy several times over, but never so small
-  // that the per-chunk table lookup and reduction epilogue show.
-  const int64_t kMax = 16384, kMin = kChunkQuantum, kTargetChunks = 4096;
+  // that the per-chunk record fetch and reduction epilogue show.
+  const int64_t kMax = RG_DEFAULT_CHUNK_ELEMS, kMin = kChunkQuantum, kTargetChunks = 4096;
   int64_t c = round_up(total / kTargetChunks + 1, kChunkQuantum);
   if (c < kMin) c = kMin;
   if (c > kMax) c = kMax;
@@ -183,8 +204,9 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
     return RG_EINVAL;
   }
   *out = nullptr;
-  if (chunk_elems < 0 || chunk_elems % kChunkQuantum != 0) {
-    set_error("rg_plan_create: chunk_elems %lld is not a multiple of %lld", (long long)chunk_elems, (long long)kChunkQuantum);
+  if (chunk_elems < 0 || chunk_elems % kChunkQuantum != 0 || chunk_elems > kMaxChunkElems) {
+    set_error("rg_plan_create: chunk_elems %lld is not a multiple of %lld in [0, %lld]", (long long)chunk_elems,
+              (long long)kChunkQuantum, (long long)kMaxChunkElems);
     return RG_EINVAL;
   }
   rg_plan* p = new (std::nothrow) rg_plan();
@@ -192,7 +214,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->device = device;
   p->n_tensors = n;
   p->host_tensors.resize((size_t)n);
-  int64_t total = 0;
+  int64_t total = 0, bytes = 0;
   for (int i = 0; i < n; ++i) {
     const int ss = elem_size(src_dtype[i]), ds = elem_size(dst_dtype[i]);
     if (ss < 0 || ds < 0 || numel[i] < 0) {
@@ -213,36 +235,33 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
       return rc;
     }
     total += numel[i];
+    bytes += numel[i] * (ss + ds);
   }
   p->total_numel = total;
+  p->total_bytes = bytes;
+  // The Infinity Cache holds 256 MiB: below that a second pass can still hit in cache.
+  p->streaming = bytes > (int64_t)256 << 20;
   p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total);
 
-  std::vector<int64_t> begin((size_t)n + 1, 0);
-  for (int i = 0; i < n; ++i) begin[(size_t)i + 1] = begin[(size_t)i] + (numel[i] + p->chunk_elems - 1) / p->chunk_elems;
-  p->n_chunks = begin[(size_t)n];
+  p->chunk_begin.assign((size_t)n + 1, 0);
+  for (int i = 0; i < n; ++i)
+    p->chunk_begin[(size_t)i + 1] = p->chunk_begin[(size_t)i] + (numel[i] + p->chunk_elems - 1) / p->chunk_elems;
+  p->n_chunks = p->chunk_begin[(size_t)n];
   if (p->n_chunks > 0x7fffffffLL) {
     set_error("rg_plan_create: %lld chunks exceed the grid limit; raise chunk_elems", (long long)p->n_chunks);
     delete p;
     return RG_EINVAL;
   }
-  std::vector<int32_t> chunk_tensor((size_t)p->n_chunks), chunk_index((size_t)p->n_chunks);
-  for (int i = 0; i < n; ++i)
-    for (int64_t c = begin[(size_t)i]; c < begin[(size_t)i + 1]; ++c) {
-      chunk_tensor[(size_t)c] = i;
-      chunk_index[(size_t)c] = (int32_t)(c - begin[(size_t)i]);
-    }
 
   // carve one device allocation
   size_t off = 0;
-  auto carve = [&off](size_t bytes) {
+  auto carve = [&off](size_t nbytes) {
     const size_t at = off;
-    off += (bytes + 255) / 256 * 256;
+    off += (nbytes + 255) / 256 * 256;
     return at;
   };
   const size_t nt = (size_t)(n > 0 ? n : 1), nc = (size_t)(p->n_chunks > 0 ? p->n_chunks : 1);
-  const size_t o_tensors = carve(nt * sizeof(TensorDesc));
-  const size_t o_ctensor = carve(nc * sizeof(int32_t));
-  const size_t o_cindex = carve(nc * sizeof(int32_t));
+  const size_t o_chunks = carve(nc * sizeof(ChunkRec));
   const size_t o_begin = carve((nt + 1) * sizeof(int64_t));
   const size_t o_sumsq = carve(nc * sizeof(double));
   const size_t o_bad = carve(nc * sizeof(int32_t));
@@ -260,9 +279,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
     return hip_fail(e, "hipMalloc(plan tables)");
   }
   char* b = p->dev_base;
-  p->d_tensors = reinterpret_cast<TensorDesc*>(b + o_tensors);
-  p->d_chunk_tensor = reinterpret_cast<int32_t*>(b + o_ctensor);
-  p->d_chunk_index = reinterpret_cast<int32_t*>(b + o_cindex);
+  p->d_chunks = reinterpret_cast<ChunkRec*>(b + o_chunks);
   p->d_tensor_chunk_begin = reinterpret_cast<int64_t*>(b + o_begin);
   p->d_chunk_sumsq = reinterpret_cast<double*>(b + o_sumsq);
   p->d_chunk_bad = reinterpret_cast<int32_t*>(b + o_bad);
@@ -272,7 +289,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->d_ticket = reinterpret_cast<unsigned int*>(b + o_ticket);
   p->d_result = reinterpret_cast<StepResult*>(b + o_result);
 
-  const size_t stage_bytes = (nt * sizeof(TensorDesc) + 255) / 256 * 256;
+  const size_t stage_bytes = (nc * sizeof(ChunkRec) + 255) / 256 * 256;
   const size_t norms_bytes = (nt * sizeof(float) + 255) / 256 * 256;
   e = hipHostMalloc(reinterpret_cast<void**>(&p->pinned), 2 * stage_bytes + 256 + norms_bytes, hipHostMallocDefault);
   if (e != hipSuccess) {
@@ -280,18 +297,18 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
     delete p;
     return hip_fail(e, "hipHostMalloc(plan staging)");
   }
-  p->stage[0] = reinterpret_cast<TensorDesc*>(p->pinned);
-  p->stage[1] = reinterpret_cast<TensorDesc*>(p->pinned + stage_bytes);
+  p->stage[0] = reinterpret_cast<ChunkRec*>(p->pinned);
+  p->stage[1] = reinterpret_cast<ChunkRec*>(p->pinned + stage_bytes);
   p->h_result = reinterpret_cast<StepResult*>(p->pinned + 2 * stage_bytes);
   p->h_norms = reinterpret_cast<float*>(p->pinned + 2 * stage_bytes + 256);
 
+  fill_chunk_records(p, p->stage[0]);
   bool ok = hipMemset(p->dev_base, 0, p->dev_bytes) == hipSuccess;
-  if (ok && n > 0) ok = hipMemcpy(p->d_tensors, p->host_tensors.data(), (size_t)n * sizeof(TensorDesc), hipMemcpyHostToDevice) == hipSuccess;
-  if (ok) ok = hipMemcpy(p->d_tensor_chunk_begin, begin.data(), begin.size() * sizeof(int64_t), hipMemcpyHostToDevice) == hipSuccess;
-  if (ok && p->n_chunks > 0) {
-    ok = hipMemcpy(p->d_chunk_tensor, chunk_tensor.data(), chunk_tensor.size() * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess &&
-         hipMemcpy(p->d_chunk_index, chunk_index.data(), chunk_index.size() * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess;
-  }
+  if (ok && p->n_chunks > 0)
+    ok = hipMemcpy(p->d_chunks, p->stage[0], (size_t)p->n_chunks * sizeof(ChunkRec), hipMemcpyHostToDevice) == hipSuccess;
+  if (ok)
+    ok = hipMemcpy(p->d_tensor_chunk_begin, p->chunk_begin.data(), p->chunk_begin.size() * sizeof(int64_t),
+                   hipMemcpyHostToDevice) == hipSuccess;
   for (int k = 0; ok && k < 2; ++k) ok = hipEventCreateWithFlags(&p->stage_done[k], hipEventDisableTiming) == hipSuccess;
   if (!ok) {
     const hipError_t last = hipGetLastError();
@@ -332,14 +349,14 @@ RG_API int rg_plan_update_pointers(rg_plan* p, const void* const* src, void* con
     if (src) p->host_tensors[(size_t)i].src = src[i];
     if (dst) p->host_tensors[(size_t)i].dst = dst[i];
   }
-  if (n == 0) return RG_OK;
+  if (p->n_chunks == 0) return RG_OK;
   DeviceGuard guard(p->device);
   const int k = p->next_stage;
   p->next_stage ^= 1;
   if (p->stage_used[k]) RG_HIP(hipEventSynchronize(p->stage_done[k]));
-  memcpy(p->stage[k], p->host_tensors.data(), (size_t)n * sizeof(TensorDesc));
+  fill_chunk_records(p, p->stage[k]);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  RG_HIP(hipMemcpyAsync(p->d_tensors, p->stage[k], (size_t)n * sizeof(TensorDesc), hipMemcpyHostToDevice, s));
+  RG_HIP(hipMemcpyAsync(p->d_chunks, p->stage[k], (size_t)p->n_chunks * sizeof(ChunkRec), hipMemcpyHostToDevice, s));
   RG_HIP(hipEventRecord(p->stage_done[k], s));
   p->stage_used[k] = true;
   return RG_OK;
@@ -350,21 +367,26 @@ RG_API int64_t rg_plan_num_chunks(const rg_plan* p) { return p ? p->n_chunks : -
 RG_API int64_t rg_plan_chunk_elems(const rg_plan* p) { return p ? p->chunk_elems : -1; }
 RG_API int64_t rg_plan_total_numel(const rg_plan* p) { return p ? p->total_numel : -1; }
 
+RG_API int rg_plan_set_streaming(rg_plan* p, int mode) {
+  if (p == nullptr || mode < -1 || mode > 1) {
+    set_error("rg_plan_set_streaming: bad arguments");
+    return RG_EINVAL;
+  }
+  p->streaming = mode < 0 ? p->total_bytes > ((int64_t)256 << 20) : mode != 0;
+  return RG_OK;
+}
+
 // ---------------------------------------------------------------------------- operations
 
 static PassArgs pass_args(const rg_plan* p, float scale) {
   PassArgs a;
-  a.tensors = p->d_tensors;
-  a.chunk_tensor = p->d_chunk_tensor;
-  a.chunk_index = p->d_chunk_index;
+  a.chunks = p->d_chunks;
   a.chunk_sumsq = p->d_chunk_sumsq;
   a.chunk_bad = p->d_chunk_bad;
   a.result = nullptr;
-  a.chunk_elems = p->chunk_elems;
   a.n_chunks = p->n_chunks;
   a.scale = scale;
   a.write_on_overflow = 0;
-  a.reverse = 0;
   a.zero_fill = 0;
   a.norm_of_source = 0;
   return a;
@@ -378,7 +400,6 @@ static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_o
   f.tensor_norm = p->d_tensor_norm;
   f.tensor_sq = p->d_tensor_sq;
   f.tensor_bad = p->d_tensor_bad;
-  f.ticket = p->d_ticket;
   f.result = p->d_result;
   f.n_tensors = p->n_tensors;
   f.max_norm = max_norm;
@@ -422,15 +443,13 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   if (p->timing_slots > 0) ev = &p->timing_events[(size_t)(p->timing_count++ % p->timing_slots) * 4];
   PassArgs a = pass_args(p, inv_scale);
   if (ev) RG_HIP(hipEventRecord(ev[0], s));
-  RG_HIP(launch_pass(kModeReduce, a, s));
+  RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
   if (ev) RG_HIP(hipEventRecord(ev[1], s));
   RG_HIP(launch_finalize(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
   if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
-  // Walk the chunks backwards: the tail of pass 1 is what the caches still hold.
-  a.reverse = 1;
-  RG_HIP(launch_pass(kModeWrite, a, s));
+  RG_HIP(launch_pass(kModeWrite, a, p->streaming, s));
   if (ev) RG_HIP(hipEventRecord(ev[3], s));
   return RG_OK;
 }
@@ -444,7 +463,7 @@ RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   }
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  RG_HIP(launch_pass(kModeReduce | kModeWrite, pass_args(p, inv_scale), s));
+  RG_HIP(launch_pass(kModeReduce | kModeWrite, pass_args(p, inv_scale), p->streaming, s));
   RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
   return RG_OK;
 }
@@ -456,7 +475,7 @@ RG_API int rg_grad_norm(rg_plan* p, void* stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, 1.0f);
   a.norm_of_source = 1;
-  RG_HIP(launch_pass(kModeReduce, a, s));
+  RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
   RG_HIP(launch_finalize(finalize_args(p, 0.0f, 1), s));
   return RG_OK;
 }
@@ -465,7 +484,7 @@ RG_API int rg_scale_cast(rg_plan* p, float scale, void* stream) {
   const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_scale_cast");
   if (rc != RG_OK) return rc;
   DeviceGuard guard(p->device);
-  RG_HIP(launch_pass(kModeWrite, pass_args(p, scale), reinterpret_cast<hipStream_t>(stream)));
+  RG_HIP(launch_pass(kModeWrite, pass_args(p, scale), p->streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }
 
@@ -475,7 +494,7 @@ RG_API int rg_zero(rg_plan* p, void* stream) {
   DeviceGuard guard(p->device);
   PassArgs a = pass_args(p, 1.0f);
   a.zero_fill = 1;
-  RG_HIP(launch_pass(kModeWrite, a, reinterpret_cast<hipStream_t>(stream)));
+  RG_HIP(launch_pass(kModeWrite, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }
 

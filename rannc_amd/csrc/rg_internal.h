@@ -11,7 +11,7 @@
 
 namespace rg {
 
-// One row of the device-side descriptor table (32 bytes).
+// One tensor pair as the caller described it (host side only).
 struct TensorDesc {
   const void* src;
   void* dst;
@@ -19,7 +19,19 @@ struct TensorDesc {
   int32_t src_dtype;
   int32_t dst_dtype;
 };
-static_assert(sizeof(TensorDesc) == 32, "descriptor row must stay 32 bytes");
+
+// One row of the device-side work table: a contiguous run of one tensor (32 bytes, so a
+// block fetches its whole work description with a single 32-byte load).
+struct ChunkRec {
+  const void* src;  // first source element of the chunk; null = the tensor has no gradient
+  void* dst;        // first destination element of the chunk
+  int32_t len;      // elements in the chunk
+  int32_t tensor;   // row of the tensor in the plan
+  int16_t src_dtype;
+  int16_t dst_dtype;
+  int32_t pad;
+};
+static_assert(sizeof(ChunkRec) == 32, "chunk record must stay 32 bytes");
 
 // Device mirror of rg_step_result, padded to 32 bytes.
 struct StepResult {
@@ -32,26 +44,33 @@ struct StepResult {
 };
 static_assert(sizeof(StepResult) == 32, "result block must stay 32 bytes");
 
-constexpr int kBlockThreads = 256;   // 4 wavefronts of 64
-constexpr int kVecElems = 8;         // elements one thread handles per vector step
-constexpr int kUnroll = 4;           // vector steps in flight per thread
-constexpr int64_t kChunkQuantum = (int64_t)kBlockThreads * kVecElems;  // 2048 elements
+// Tunables (overridable at build time for experiments).
+#ifndef RG_ELEMS_PER_THREAD_ITER
+#define RG_ELEMS_PER_THREAD_ITER 32
+#endif
+#ifndef RG_ALIGN_BYTES
+#define RG_ALIGN_BYTES 128
+#endif
+#ifndef RG_DEFAULT_CHUNK_ELEMS
+#define RG_DEFAULT_CHUNK_ELEMS 16384
+#endif
+constexpr int kBlockThreads = 256;                               // 4 wavefronts of 64
+constexpr int kElemsPerThreadIter = RG_ELEMS_PER_THREAD_ITER;    // elements a thread has in flight per loop iteration
+constexpr unsigned kAlignBytes = RG_ALIGN_BYTES;                 // per-chunk peel of the written (or read-only) side
+constexpr int64_t kChunkQuantum = 2048;    // chunk sizes are multiples of this many elements
+constexpr int64_t kMaxChunkElems = 1 << 20;
 
 // Pass selection for the chunk kernel.
 enum : int { kModeReduce = 1, kModeWrite = 2 };
 
 struct PassArgs {
-  const TensorDesc* tensors;
-  const int32_t* chunk_tensor;   // [n_chunks] row of the descriptor table
-  const int32_t* chunk_index;    // [n_chunks] which chunk of that tensor
+  const ChunkRec* chunks;        // [n_chunks]
   double* chunk_sumsq;           // [n_chunks] written when reducing
   int32_t* chunk_bad;            // [n_chunks] written when reducing
   const StepResult* result;      // non-null: take coef / overflow gate from the device
-  int64_t chunk_elems;
   int64_t n_chunks;
   float scale;
   int32_t write_on_overflow;
-  int32_t reverse;               // visit chunks last to first
   int32_t zero_fill;             // write pass: ignore the sources, store zeros
   int32_t norm_of_source;        // reduce pass: measure the source as stored (no rounding to dst)
 };
@@ -63,14 +82,14 @@ struct FinalizeArgs {
   float* tensor_norm;                 // [n_tensors]
   double* tensor_sq;                  // [n_tensors]
   int32_t* tensor_bad;                // [n_tensors]
-  unsigned int* ticket;
   StepResult* result;
   int32_t n_tensors;
   float max_norm;
   int32_t ignore_overflow;  // overflow is reported but neither gates the clip nor the write
 };
 
-hipError_t launch_pass(int mode, const PassArgs& a, hipStream_t stream);
+// streaming: nontemporal loads/stores (data far larger than the caches).
+hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
 

@@ -1,54 +1,83 @@
 // gfx950 kernels of libranncgrad.
 //
 // One "pass" kernel serves every per-step operation.  The grid is the plan's chunk list:
-// block b looks up (tensor, chunk-of-tensor) in the device-side table, so a launch covers
-// thousands of tensors of any size mix.  A chunk is a contiguous run of at most
-// chunk_elems elements of one tensor; inside it a thread moves 8 elements per step with
-// 128-bit accesses.  The side that is written (or, for a read-only pass, the side that is
-// read) is peeled to a 16-byte boundary per chunk; the other side is accessed at its
-// natural element alignment, which gfx950 serves with the same 128-bit instruction.
+// block b reads one 32-byte chunk record (source pointer, destination pointer, length,
+// element types) and streams that chunk, so a launch covers thousands of tensors of any
+// size mix and a block needs a single table lookup before its first data load.
 //
-// The pass is purely bandwidth bound (a few ALU ops per element), so there is no LDS
-// staging and no MFMA: LDS is used only for the 4-wavefront combine of the partial sums.
+// Inside a chunk every load and store instruction is contiguous across the wavefront: a
+// lane moves E consecutive elements per instruction, E = 4 when either side is fp32 and 8
+// otherwise, so the wider side always moves 16 bytes per lane (1 KiB per wavefront
+// instruction) and the narrower side 8.  The side that is written (for a read-only pass,
+// the side that is read) is peeled to a 128-byte boundary per chunk, so streaming stores
+// cover whole lines; the other side is accessed at its natural element alignment, which
+// gfx950 serves with the same instructions.
+//
+// Plans whose data is far larger than the caches use nontemporal loads and stores: measured
+// on MI355X that lifts a read-only pass from 6.3 to 7.1 TB/s, and nontemporal stores keep
+// dirty lines from lingering in L2 / Infinity Cache where their write-back would slow the
+// next kernel's reads.  Small plans use plain accesses so the second pass hits in cache.
+//
+// The work is purely bandwidth bound (a few ALU ops per element): no LDS staging and no
+// MFMA.  LDS is used only for the 4-wavefront combine of the partial sums.
 #include "rg_internal.h"
 
 namespace rg {
 namespace {
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-// 16-byte vectors at element alignment (2 or 4 bytes).
-struct __attribute__((packed, aligned(2))) V16A2 { u32x4 v; };
-struct __attribute__((packed, aligned(4))) V16A4 { u32x4 v; };
+// Vector types whose alignment is only that of one element (2 or 4 bytes).
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
 
 template <int DT> struct ElemSize { static constexpr int value = 2; };
 template <> struct ElemSize<RG_F32> { static constexpr int value = 4; };
 
-// Eight elements in their memory representation.
-template <int DT> struct Raw { u32x4 a; };
-template <> struct Raw<RG_F32> { u32x4 a, b; };
+// E elements of type DT as they sit in memory: 8 or 16 bytes.
+template <int DT, int E> struct Raw;
+template <> struct Raw<RG_F32, 4> { u32x4 v; };
+template <> struct Raw<RG_F16, 4> { u32x2 v; };
+template <> struct Raw<RG_BF16, 4> { u32x2 v; };
+template <> struct Raw<RG_F16, 8> { u32x4 v; };
+template <> struct Raw<RG_BF16, 8> { u32x4 v; };
 
-template <int DT> __device__ __forceinline__ Raw<DT> load_raw(const char* p) {
-  Raw<DT> r;
-  r.a = reinterpret_cast<const V16A2*>(p)->v;
-  return r;
+// Loads at element alignment.
+template <bool NT> __device__ __forceinline__ u32x4 ld16_a4(const char* p) {
+  return NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4_a4*>(p)) : *reinterpret_cast<const u32x4_a4*>(p);
 }
-template <> __device__ __forceinline__ Raw<RG_F32> load_raw<RG_F32>(const char* p) {
-  Raw<RG_F32> r;
-  r.a = reinterpret_cast<const V16A4*>(p)->v;
-  r.b = reinterpret_cast<const V16A4*>(p + 16)->v;
-  return r;
+template <bool NT> __device__ __forceinline__ u32x4 ld16_a2(const char* p) {
+  return NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4_a2*>(p)) : *reinterpret_cast<const u32x4_a2*>(p);
+}
+template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
+  return NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x2_a2*>(p)) : *reinterpret_cast<const u32x2_a2*>(p);
+}
+// Stores are aligned to their own size (the chunk head is peeled for that).
+template <bool NT> __device__ __forceinline__ void st16(char* p, u32x4 v) {
+  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+  else *reinterpret_cast<u32x4*>(p) = v;
+}
+template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
+  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+  else *reinterpret_cast<u32x2*>(p) = v;
 }
 
-// Stores are always 16-byte aligned (the chunk head is peeled for that).
-template <int DT> __device__ __forceinline__ void store_raw(char* p, const Raw<DT>& r) {
-  *reinterpret_cast<u32x4*>(p) = r.a;
-}
-template <> __device__ __forceinline__ void store_raw<RG_F32>(char* p, const Raw<RG_F32>& r) {
-  *reinterpret_cast<u32x4*>(p) = r.a;
-  *reinterpret_cast<u32x4*>(p + 16) = r.b;
-}
+template <int DT, int E, bool NT> struct Mem;
+template <bool NT> struct Mem<RG_F32, 4, NT> {
+  static __device__ __forceinline__ Raw<RG_F32, 4> load(const char* p) { return {ld16_a4<NT>(p)}; }
+  static __device__ __forceinline__ void store(char* p, const Raw<RG_F32, 4>& r) { st16<NT>(p, r.v); }
+};
+template <int DT, bool NT> struct Mem<DT, 4, NT> {   // 16-bit types, 4 elements = 8 bytes
+  static __device__ __forceinline__ Raw<DT, 4> load(const char* p) { return {ld8_a2<NT>(p)}; }
+  static __device__ __forceinline__ void store(char* p, const Raw<DT, 4>& r) { st8<NT>(p, r.v); }
+};
+template <int DT, bool NT> struct Mem<DT, 8, NT> {   // 16-bit types, 8 elements = 16 bytes
+  static __device__ __forceinline__ Raw<DT, 8> load(const char* p) { return {ld16_a2<NT>(p)}; }
+  static __device__ __forceinline__ void store(char* p, const Raw<DT, 8>& r) { st16<NT>(p, r.v); }
+};
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
@@ -63,53 +92,51 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
   return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f);
 }
 
-template <int DT> __device__ __forceinline__ void unpack(const Raw<DT>& r, float (&f)[8]);
-template <> __device__ __forceinline__ void unpack<RG_F32>(const Raw<RG_F32>& r, float (&f)[8]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    f[j] = __uint_as_float(r.a[j]);
-    f[4 + j] = __uint_as_float(r.b[j]);
-  }
+template <int DT> __device__ __forceinline__ void unpack_word(uint32_t w, float& lo, float& hi);
+template <> __device__ __forceinline__ void unpack_word<RG_F16>(uint32_t w, float& lo, float& hi) {
+  const f16x2 h = __builtin_bit_cast(f16x2, w);   // bit_cast needs a scalar, not a vector-element lvalue
+  lo = (float)h.x;
+  hi = (float)h.y;
 }
-template <> __device__ __forceinline__ void unpack<RG_F16>(const Raw<RG_F16>& r, float (&f)[8]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const unsigned int w = r.a[j];  // bit_cast must see a scalar, not a vector-element lvalue
-    const f16x2 h = __builtin_bit_cast(f16x2, w);
-    f[2 * j] = (float)h.x;
-    f[2 * j + 1] = (float)h.y;
-  }
+template <> __device__ __forceinline__ void unpack_word<RG_BF16>(uint32_t w, float& lo, float& hi) {
+  lo = __uint_as_float(w << 16);
+  hi = __uint_as_float(w & 0xffff0000u);
 }
-template <> __device__ __forceinline__ void unpack<RG_BF16>(const Raw<RG_BF16>& r, float (&f)[8]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    f[2 * j] = __uint_as_float(r.a[j] << 16);
-    f[2 * j + 1] = __uint_as_float(r.a[j] & 0xffff0000u);
-  }
+template <int DT> __device__ __forceinline__ uint32_t pack_word(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack_word<RG_F16>(float lo, float hi) {
+  return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+}
+template <> __device__ __forceinline__ uint32_t pack_word<RG_BF16>(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
 }
 
-template <int DT> __device__ __forceinline__ Raw<DT> pack(const float (&f)[8]);
-template <> __device__ __forceinline__ Raw<RG_F32> pack<RG_F32>(const float (&f)[8]) {
-  Raw<RG_F32> r;
+template <int DT, int E> struct Codec {   // 16-bit types
+  static __device__ __forceinline__ void unpack(const Raw<DT, E>& r, float (&f)[E]) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    r.a[j] = __float_as_uint(f[j]);
-    r.b[j] = __float_as_uint(f[4 + j]);
+    for (int j = 0; j < E / 2; ++j) {
+      const uint32_t w = r.v[j];
+      unpack_word<DT>(w, f[2 * j], f[2 * j + 1]);
+    }
   }
-  return r;
-}
-template <> __device__ __forceinline__ Raw<RG_F16> pack<RG_F16>(const float (&f)[8]) {
-  Raw<RG_F16> r;
+  static __device__ __forceinline__ Raw<DT, E> pack(const float (&f)[E]) {
+    Raw<DT, E> r;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) r.a[j] = f32_to_f16_bits(f[2 * j]) | (f32_to_f16_bits(f[2 * j + 1]) << 16);
-  return r;
-}
-template <> __device__ __forceinline__ Raw<RG_BF16> pack<RG_BF16>(const float (&f)[8]) {
-  Raw<RG_BF16> r;
+    for (int j = 0; j < E / 2; ++j) r.v[j] = pack_word<DT>(f[2 * j], f[2 * j + 1]);
+    return r;
+  }
+};
+template <> struct Codec<RG_F32, 4> {
+  static __device__ __forceinline__ void unpack(const Raw<RG_F32, 4>& r, float (&f)[4]) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) r.a[j] = f32_to_bf16_bits(f[2 * j]) | (f32_to_bf16_bits(f[2 * j + 1]) << 16);
-  return r;
-}
+    for (int j = 0; j < 4; ++j) f[j] = __uint_as_float(r.v[j]);
+  }
+  static __device__ __forceinline__ Raw<RG_F32, 4> pack(const float (&f)[4]) {
+    Raw<RG_F32, 4> r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.v[j] = __float_as_uint(f[j]);
+    return r;
+  }
+};
 
 // The value as it reads back from a destination of type DT.
 template <int DT> __device__ __forceinline__ float round_dst(float v) { return v; }
@@ -147,130 +174,127 @@ template <> __device__ __forceinline__ bool nonfinite_at<RG_BF16>(const char* p)
   return (*reinterpret_cast<const unsigned short*>(p) & 0x7f80u) == 0x7f80u;
 }
 
-// v = round_dst(x * scale); sum += v^2; out = round_dst(v * coef).
+// One chunk.  v = round_dst(x * scale); sum += v^2; out = round_dst(v * coef).
 // coef is 1 when nothing is clipped: v * 1 is v bit for bit, so no branch is needed.
-// Two separate multiplies, never fused or reassociated (the file is built with
+// The two multiplies are never fused or reassociated (the file is built with
 // -ffp-contract=off), so the result matches `x.float() * inv_scale` then `mul_(coef)`.
-template <int S, int D, int MODE>
-__device__ __forceinline__ void compute8(const Raw<S>& in, Raw<D>& out, float (&acc)[8], float scale,
-                                         float coef) {
-  float f[8];
-  unpack<S>(in, f);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float v = round_dst<D>(f[j] * scale);
-    if (MODE & kModeReduce) acc[j] = __builtin_fmaf(v, v, acc[j]);
-    if (MODE & kModeWrite) f[j] = round_dst<D>(v * coef);
-  }
-  if (MODE & kModeWrite) out = pack<D>(f);
-}
-
-template <int S, int D, int MODE>
-__device__ __forceinline__ void process_chunk(const char* sp, char* dp, int64_t len, float scale,
-                                              float coef, bool raw_copy, float (&acc)[8]) {
+template <int S, int D, int MODE, bool NT>
+__device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len, float scale, float coef,
+                                              bool raw_copy, float (&acc)[8]) {
   constexpr int SS = ElemSize<S>::value;
   constexpr int DS = ElemSize<D>::value;
   constexpr bool kWrite = (MODE & kModeWrite) != 0;
+  constexpr bool kReduce = (MODE & kModeReduce) != 0;
+  constexpr int E = (SS == 4 || (kWrite && DS == 4)) ? 4 : 8;   // elements per lane per instruction
+  constexpr int U = kElemsPerThreadIter / E;                    // instructions in flight per lane
   constexpr int AS = kWrite ? DS : SS;
   const uintptr_t a = kWrite ? reinterpret_cast<uintptr_t>(dp) : reinterpret_cast<uintptr_t>(sp);
-  int64_t head = (int64_t)(((16u - (unsigned)(a & 15u)) & 15u) / (unsigned)AS);
+  int head = (int)(((kAlignBytes - (unsigned)(a & (kAlignBytes - 1))) & (kAlignBytes - 1)) / (unsigned)AS);
   if (head > len) head = len;
-  const int64_t nvec = (len - head) / kVecElems;
-  const int64_t tail0 = head + nvec * kVecElems;
+  const int nbody = (len - head) / E * E;
+  const int tail0 = head + nbody;
   const int tid = threadIdx.x;
 
-  // Unaligned head (< 8 elements) and ragged tail (< 8 elements): one element per thread.
-  const int nscalar = (int)(head + (len - tail0));
+  // Unaligned head (< 128 bytes) and ragged tail (< E elements): one element per thread.
+  const int nscalar = head + (len - tail0);
   if (tid < nscalar) {
-    const int64_t i = tid < head ? (int64_t)tid : tail0 + (tid - head);
+    const int i = tid < head ? tid : tail0 + (tid - head);
     if (S == D && raw_copy) {
-      if (SS == 4) *reinterpret_cast<uint32_t*>(dp + i * 4) = *reinterpret_cast<const uint32_t*>(sp + i * 4);
-      else *reinterpret_cast<unsigned short*>(dp + i * 2) = *reinterpret_cast<const unsigned short*>(sp + i * 2);
+      if (SS == 4) *reinterpret_cast<uint32_t*>(dp + (size_t)i * 4) = *reinterpret_cast<const uint32_t*>(sp + (size_t)i * 4);
+      else *reinterpret_cast<unsigned short*>(dp + (size_t)i * 2) = *reinterpret_cast<const unsigned short*>(sp + (size_t)i * 2);
     } else {
-      const float v = round_dst<D>(load1<S>(sp + i * SS) * scale);
-      if (MODE & kModeReduce) acc[0] = __builtin_fmaf(v, v, acc[0]);
-      if (kWrite) store1<D>(dp + i * DS, v * coef);
+      const float v = round_dst<D>(load1<S>(sp + (size_t)i * SS) * scale);
+      if (kReduce) acc[0] = __builtin_fmaf(v, v, acc[0]);
+      if (kWrite) store1<D>(dp + (size_t)i * DS, v * coef);
     }
   }
 
-  const char* sb = sp + head * SS;
-  char* db = dp + head * DS;
-  constexpr int64_t kStep = (int64_t)kBlockThreads * kUnroll;
-  int64_t v0 = 0;
-  for (; v0 + kStep <= nvec; v0 += kStep) {
-    Raw<S> in[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      in[u] = load_raw<S>(sb + (v0 + u * kBlockThreads + tid) * (kVecElems * SS));
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int64_t v = v0 + u * kBlockThreads + tid;
-      if (S == D && raw_copy) {
-        Raw<D> out;
-        __builtin_memcpy(&out, &in[u], sizeof(out));
-        store_raw<D>(db + v * (kVecElems * DS), out);
-      } else {
-        Raw<D> out;
-        compute8<S, D, MODE>(in[u], out, acc, scale, coef);
-        if (kWrite) store_raw<D>(db + v * (kVecElems * DS), out);
+  const char* sb = sp + (size_t)head * SS;
+  char* db = dp + (size_t)head * DS;
+  constexpr int kIter = kBlockThreads * E * U;   // elements per block iteration
+
+  // All U loads of an iteration are issued back to back with no branch between them, so
+  // they are all in flight together.  `valid` only guards what is accumulated and stored.
+  auto consume = [&](const Raw<S, E>& in, int e, bool valid) {
+    bool copied = false;
+    if constexpr (S == D && kWrite) {
+      if (raw_copy) {
+        if (valid) Mem<D, E, NT>::store(db + (size_t)e * DS, in);
+        copied = true;
       }
     }
-  }
-  if (v0 < nvec) {
-    Raw<S> in[kUnroll];
+    if (!copied) {
+      float f[E];
+      Codec<S, E>::unpack(in, f);
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int64_t v = v0 + u * kBlockThreads + tid;
-      if (v < nvec) in[u] = load_raw<S>(sb + v * (kVecElems * SS));
-    }
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int64_t v = v0 + u * kBlockThreads + tid;
-      if (v < nvec) {
-        if (S == D && raw_copy) {
-          Raw<D> out;
-          __builtin_memcpy(&out, &in[u], sizeof(out));
-          store_raw<D>(db + v * (kVecElems * DS), out);
-        } else {
-          Raw<D> out;
-          compute8<S, D, MODE>(in[u], out, acc, scale, coef);
-          if (kWrite) store_raw<D>(db + v * (kVecElems * DS), out);
+      for (int j = 0; j < E; ++j) {
+        float v = round_dst<D>(f[j] * scale);
+        if (kReduce) {
+          const float q = valid ? v : 0.0f;
+          acc[j & 7] = __builtin_fmaf(q, q, acc[j & 7]);
         }
+        if (kWrite) f[j] = round_dst<D>(v * coef);
       }
+      if constexpr (kWrite) {
+        if (valid) Mem<D, E, NT>::store(db + (size_t)e * DS, Codec<D, E>::pack(f));
+      }
+    }
+  };
+
+  int base = 0;
+  for (; base + kIter <= nbody; base += kIter) {
+    Raw<S, E> in[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) in[u] = Mem<S, E, NT>::load(sb + (size_t)(base + (u * kBlockThreads + tid) * E) * SS);
+#pragma unroll
+    for (int u = 0; u < U; ++u) consume(in[u], base + (u * kBlockThreads + tid) * E, true);
+  }
+  if (base < nbody) {
+    // Last, partial iteration: lanes past the end re-read the final vector (an address that
+    // is certainly valid) so the loads stay unconditional, and are masked afterwards.
+    Raw<S, E> in[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int e = base + (u * kBlockThreads + tid) * E;
+      in[u] = Mem<S, E, NT>::load(sb + (size_t)(e < nbody ? e : nbody - E) * SS);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int e = base + (u * kBlockThreads + tid) * E;
+      consume(in[u], e, e < nbody);
     }
   }
 }
 
 // Zero `nbytes` bytes at p (p and nbytes are multiples of 2).
-__device__ __forceinline__ void zero_range(char* p, int64_t nbytes) {
+template <bool NT>
+__device__ __forceinline__ void zero_range(char* p, int nbytes) {
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
-  int64_t head = (int64_t)((16u - (unsigned)(a & 15u)) & 15u);
+  int head = (int)((kAlignBytes - (unsigned)(a & (kAlignBytes - 1))) & (kAlignBytes - 1));
   if (head > nbytes) head = nbytes;
-  const int64_t nvec = (nbytes - head) / 16;
-  const int64_t tail0 = head + nvec * 16;
+  const int nvec = (nbytes - head) / 16;
+  const int tail0 = head + nvec * 16;
   const int tid = threadIdx.x;
-  const int nscalar = (int)((head + (nbytes - tail0)) / 2);
+  const int nscalar = (head + (nbytes - tail0)) / 2;
   if (tid < nscalar) {
-    const int64_t off = tid < head / 2 ? (int64_t)tid * 2 : tail0 + ((int64_t)tid - head / 2) * 2;
+    const int off = tid < head / 2 ? tid * 2 : tail0 + (tid - head / 2) * 2;
     *reinterpret_cast<unsigned short*>(p + off) = 0;
   }
   const u32x4 z = {0u, 0u, 0u, 0u};
-  for (int64_t v = tid; v < nvec; v += kBlockThreads) *reinterpret_cast<u32x4*>(p + head + v * 16) = z;
+  for (int v = tid; v < nvec; v += kBlockThreads) st16<NT>(p + head + (size_t)v * 16, z);
 }
 
 template <int S>
-__device__ __forceinline__ int rescan_nonfinite(const char* sp, int64_t len) {
+__device__ __forceinline__ int rescan_nonfinite(const char* sp, int len) {
   int bad = 0;
-  for (int64_t i = threadIdx.x; i < len; i += kBlockThreads)
-    bad |= nonfinite_at<S>(sp + i * ElemSize<S>::value) ? 1 : 0;
+  for (int i = threadIdx.x; i < len; i += kBlockThreads)
+    bad |= nonfinite_at<S>(sp + (size_t)i * ElemSize<S>::value) ? 1 : 0;
   return bad;
 }
 
-template <int MODE>
+template <int MODE, bool NT>
 __global__ __launch_bounds__(kBlockThreads) void pass_kernel(PassArgs a) {
-  int64_t c = blockIdx.x;
-  if (a.reverse) c = a.n_chunks - 1 - c;
-
+  const int64_t c = blockIdx.x;
   float coef = 1.0f;
   if (a.result != nullptr) {
     // Values produced by the finalize kernel earlier on the same stream.
@@ -278,32 +302,28 @@ __global__ __launch_bounds__(kBlockThreads) void pass_kernel(PassArgs a) {
     coef = a.result->coef;
   }
 
-  const TensorDesc t = a.tensors[a.chunk_tensor[c]];
-  const int64_t start = (int64_t)a.chunk_index[c] * a.chunk_elems;
-  int64_t len = t.numel - start;
-  if (len > a.chunk_elems) len = a.chunk_elems;
-
-  const int ss = t.src_dtype == RG_F32 ? 4 : 2;
-  const int ds = t.dst_dtype == RG_F32 ? 4 : 2;
-  const char* sp = reinterpret_cast<const char*>(t.src) + start * ss;
-  char* dp = reinterpret_cast<char*>(t.dst) + start * ds;
+  const ChunkRec rec = a.chunks[c];
+  const int len = rec.len;
+  const char* sp = reinterpret_cast<const char*>(rec.src);
+  char* dp = reinterpret_cast<char*>(rec.dst);
+  const int src_kind = rec.src_dtype;
+  const int dst_kind = a.norm_of_source ? rec.src_dtype : rec.dst_dtype;
   const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale == 1.0f;
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const int dst_kind = a.norm_of_source ? t.src_dtype : t.dst_dtype;
-  if (t.src == nullptr || a.zero_fill) {
-    if (MODE & kModeWrite) zero_range(dp, len * ds);
+  if (sp == nullptr || a.zero_fill) {
+    if (MODE & kModeWrite) zero_range<NT>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
   } else {
-    switch (t.src_dtype * 3 + dst_kind) {
-      case RG_F32 * 3 + RG_F32: process_chunk<RG_F32, RG_F32, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      case RG_F32 * 3 + RG_F16: process_chunk<RG_F32, RG_F16, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      case RG_F32 * 3 + RG_BF16: process_chunk<RG_F32, RG_BF16, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      case RG_F16 * 3 + RG_F32: process_chunk<RG_F16, RG_F32, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      case RG_F16 * 3 + RG_F16: process_chunk<RG_F16, RG_F16, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      case RG_F16 * 3 + RG_BF16: process_chunk<RG_F16, RG_BF16, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      case RG_BF16 * 3 + RG_F32: process_chunk<RG_BF16, RG_F32, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      case RG_BF16 * 3 + RG_F16: process_chunk<RG_BF16, RG_F16, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
-      default: process_chunk<RG_BF16, RG_BF16, MODE>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+    switch (src_kind * 3 + dst_kind) {
+      case RG_F32 * 3 + RG_F32: process_chunk<RG_F32, RG_F32, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      case RG_F32 * 3 + RG_F16: process_chunk<RG_F32, RG_F16, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      case RG_F32 * 3 + RG_BF16: process_chunk<RG_F32, RG_BF16, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      case RG_F16 * 3 + RG_F32: process_chunk<RG_F16, RG_F32, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      case RG_F16 * 3 + RG_F16: process_chunk<RG_F16, RG_F16, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      case RG_F16 * 3 + RG_BF16: process_chunk<RG_F16, RG_BF16, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      case RG_BF16 * 3 + RG_F32: process_chunk<RG_BF16, RG_F32, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      case RG_BF16 * 3 + RG_F16: process_chunk<RG_BF16, RG_F16, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
+      default: process_chunk<RG_BF16, RG_BF16, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
     }
   }
 
@@ -324,9 +344,9 @@ __global__ __launch_bounds__(kBlockThreads) void pass_kernel(PassArgs a) {
     int bad = 0;
     if (!(fabs(total) <= 1.79769313486231570e308)) {
       int mine = 0;
-      if (t.src != nullptr) {
-        if (t.src_dtype == RG_F32) mine = rescan_nonfinite<RG_F32>(sp, len);
-        else if (t.src_dtype == RG_F16) mine = rescan_nonfinite<RG_F16>(sp, len);
+      if (sp != nullptr) {
+        if (src_kind == RG_F32) mine = rescan_nonfinite<RG_F32>(sp, len);
+        else if (src_kind == RG_F16) mine = rescan_nonfinite<RG_F16>(sp, len);
         else mine = rescan_nonfinite<RG_BF16>(sp, len);
       }
       bad = __syncthreads_or(mine);
@@ -338,67 +358,81 @@ __global__ __launch_bounds__(kBlockThreads) void pass_kernel(PassArgs a) {
   }
 }
 
-// Wavefront w of the grid reduces tensor w's chunk sums (lane-strided, then a fixed
-// shuffle tree) to n_t = float(sqrt(sum)).  The last block to finish then adds
-// double(n_t)^2 over all tensors in a fixed order and derives the clip decision.
-__global__ __launch_bounds__(kBlockThreads) void finalize_kernel(FinalizeArgs a) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int t = blockIdx.x * (kBlockThreads / 64) + wave;
-  if (t < a.n_tensors) {
-    double s = 0.0;
-    int bad = 0;
-    const int64_t end = a.tensor_chunk_begin[t + 1];
-    for (int64_t c = a.tensor_chunk_begin[t] + lane; c < end; c += 64) {
-      s += a.chunk_sumsq[c];
-      bad |= a.chunk_bad[c];
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      s += __shfl_down(s, off);
-      bad |= __shfl_down(bad, off);
-    }
-    if (lane == 0) {
-      const float n = (float)sqrt(s);
-      a.tensor_norm[t] = n;
-      a.tensor_sq[t] = (double)n * (double)n;
-      a.tensor_bad[t] = bad;
-    }
-  }
-
-  __shared__ int is_last;
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const unsigned prev = atomicAdd(a.ticket, 1u);
-    is_last = (prev == gridDim.x - 1) ? 1 : 0;
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-
-  double s = 0.0;
-  int bad = 0;
-  for (int i = threadIdx.x; i < a.n_tensors; i += kBlockThreads) {
-    s += a.tensor_sq[i];
-    bad |= a.tensor_bad[i];
-  }
+// Fixed-order sum of one value per thread over the block: shuffle tree inside each
+// wavefront, then the wavefront totals through LDS in index order.
+__device__ __forceinline__ void block_sum_or(double& s, int& bad, double* lds_sum, int* lds_bad) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     s += __shfl_down(s, off);
     bad |= __shfl_down(bad, off);
   }
-  __shared__ double wave_sum[kBlockThreads / 64];
-  __shared__ int wave_bad[kBlockThreads / 64];
-  if (lane == 0) {
-    wave_sum[wave] = s;
-    wave_bad[wave] = bad;
+  if ((threadIdx.x & 63) == 0) {
+    lds_sum[threadIdx.x >> 6] = s;
+    lds_bad[threadIdx.x >> 6] = bad;
   }
   __syncthreads();
+  s = (lds_sum[0] + lds_sum[1]) + (lds_sum[2] + lds_sum[3]);
+  bad = lds_bad[0] | lds_bad[1] | lds_bad[2] | lds_bad[3];
+  __syncthreads();
+}
+
+// Block t reduces tensor t's chunk sums (thread-strided with four independent loads in
+// flight, then a fixed tree) to n_t = float(sqrt(sum)).
+__global__ __launch_bounds__(kBlockThreads) void finalize_tensors_kernel(FinalizeArgs a) {
+  __shared__ double lds_sum[kBlockThreads / 64];
+  __shared__ int lds_bad[kBlockThreads / 64];
+  const int t = blockIdx.x;
+  double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+  int bad = 0;
+  const int64_t end = a.tensor_chunk_begin[t + 1];
+  int64_t c = a.tensor_chunk_begin[t] + threadIdx.x;
+  for (; c + 3 * kBlockThreads < end; c += 4 * kBlockThreads) {
+    const double v0 = a.chunk_sumsq[c], v1 = a.chunk_sumsq[c + kBlockThreads];
+    const double v2 = a.chunk_sumsq[c + 2 * kBlockThreads], v3 = a.chunk_sumsq[c + 3 * kBlockThreads];
+    const int b0 = a.chunk_bad[c], b1 = a.chunk_bad[c + kBlockThreads];
+    const int b2 = a.chunk_bad[c + 2 * kBlockThreads], b3 = a.chunk_bad[c + 3 * kBlockThreads];
+    s0 += v0; s1 += v1; s2 += v2; s3 += v3;
+    bad |= b0 | b1 | b2 | b3;
+  }
+  for (; c < end; c += kBlockThreads) {
+    s0 += a.chunk_sumsq[c];
+    bad |= a.chunk_bad[c];
+  }
+  double s = (s0 + s1) + (s2 + s3);
+  block_sum_or(s, bad, lds_sum, lds_bad);
   if (threadIdx.x == 0) {
-    const double total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
-    const int overflow = (wave_bad[0] | wave_bad[1] | wave_bad[2] | wave_bad[3]) != 0 ? 1 : 0;
-    const double norm = sqrt(total);
+    const float n = (float)sqrt(s);
+    a.tensor_norm[t] = n;
+    a.tensor_sq[t] = (double)n * (double)n;
+    a.tensor_bad[t] = bad;
+  }
+}
+
+// One block adds double(n_t)^2 over all tensors in a fixed order and derives the clip
+// decision.  It runs as its own launch after finalize_tensors_kernel: a kernel boundary
+// is a far cheaper device-wide barrier here than per-block fences, whose L2 write-back
+// across the eight XCDs cost about 30 us for a few hundred blocks.
+__global__ __launch_bounds__(kBlockThreads) void finalize_total_kernel(FinalizeArgs a) {
+  __shared__ double lds_sum[kBlockThreads / 64];
+  __shared__ int lds_bad[kBlockThreads / 64];
+  double s0 = 0.0, s1 = 0.0;
+  int bad = 0;
+  int i = threadIdx.x;
+  for (; i + kBlockThreads < a.n_tensors; i += 2 * kBlockThreads) {
+    const double v0 = a.tensor_sq[i], v1 = a.tensor_sq[i + kBlockThreads];
+    const int b0 = a.tensor_bad[i], b1 = a.tensor_bad[i + kBlockThreads];
+    s0 += v0; s1 += v1;
+    bad |= b0 | b1;
+  }
+  for (; i < a.n_tensors; i += kBlockThreads) {
+    s0 += a.tensor_sq[i];
+    bad |= a.tensor_bad[i];
+  }
+  double s = s0 + s1;
+  block_sum_or(s, bad, lds_sum, lds_bad);
+  if (threadIdx.x == 0) {
+    const int overflow = bad != 0 ? 1 : 0;
+    const double norm = sqrt(s);
     const double g = norm + 1e-6;
     const bool gate = overflow != 0 && a.ignore_overflow == 0;
     const bool clip = a.max_norm > 0.0f && !gate && (g > (double)a.max_norm);
@@ -407,7 +441,6 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_kernel(FinalizeArgs a)
     a.result->overflow = overflow;
     a.result->clipped = clip ? 1 : 0;
     a.result->skipped = gate ? 1 : 0;
-    *a.ticket = 0u;
   }
 }
 
@@ -425,24 +458,29 @@ __global__ __launch_bounds__(kBlockThreads) void fill_zero_kernel(char* p, int64
   for (int64_t v = gtid; v < nvec; v += nthreads) *reinterpret_cast<u32x4*>(p + head + v * 16) = z;
 }
 
+template <int MODE>
+void launch_mode(const PassArgs& a, bool streaming, hipStream_t stream) {
+  const dim3 grid((unsigned)a.n_chunks), block(kBlockThreads);
+  if (streaming) hipLaunchKernelGGL((pass_kernel<MODE, true>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((pass_kernel<MODE, false>), grid, block, 0, stream, a);
+}
+
 }  // namespace
 
-hipError_t launch_pass(int mode, const PassArgs& a, hipStream_t stream) {
+hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream) {
   if (a.n_chunks <= 0) return hipSuccess;
-  const dim3 grid((unsigned)a.n_chunks), block(kBlockThreads);
   switch (mode) {
-    case kModeReduce: hipLaunchKernelGGL(pass_kernel<kModeReduce>, grid, block, 0, stream, a); break;
-    case kModeWrite: hipLaunchKernelGGL(pass_kernel<kModeWrite>, grid, block, 0, stream, a); break;
-    default: hipLaunchKernelGGL(pass_kernel<kModeReduce | kModeWrite>, grid, block, 0, stream, a); break;
+    case kModeReduce: launch_mode<kModeReduce>(a, streaming, stream); break;
+    case kModeWrite: launch_mode<kModeWrite>(a, streaming, stream); break;
+    default: launch_mode<kModeReduce | kModeWrite>(a, streaming, stream); break;
   }
   return hipGetLastError();
 }
 
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream) {
-  const int waves_per_block = kBlockThreads / 64;
-  int blocks = (a.n_tensors + waves_per_block - 1) / waves_per_block;
-  if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(finalize_kernel, dim3((unsigned)blocks), dim3(kBlockThreads), 0, stream, a);
+  if (a.n_tensors > 0)
+    hipLaunchKernelGGL(finalize_tensors_kernel, dim3((unsigned)a.n_tensors), dim3(kBlockThreads), 0, stream, a);
+  hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
   return hipGetLastError();
 }
 
