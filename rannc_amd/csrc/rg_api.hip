@@ -2,6 +2,7 @@
 // device) and the extern "C" entry points declared in include/ranncgrad.h.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <new>
@@ -69,6 +70,7 @@ struct rg_plan {
   int64_t chunk_elems = 0;
   int64_t n_chunks = 0;
   bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
+  int64_t write_tile_elems = kWriteTileElems;
   std::vector<TensorDesc> host_tensors;
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
 
@@ -242,6 +244,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   // The Infinity Cache holds 256 MiB: below that a second pass can still hit in cache.
   p->streaming = bytes > (int64_t)256 << 20;
   p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total);
+  if (const char* env = getenv("RG_WRITE_TILE_ELEMS")) p->write_tile_elems = atoll(env);
 
   p->chunk_begin.assign((size_t)n + 1, 0);
   for (int i = 0; i < n; ++i)
@@ -385,6 +388,8 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   a.chunk_bad = p->d_chunk_bad;
   a.result = nullptr;
   a.n_chunks = p->n_chunks;
+  a.tile_elems = (int32_t)p->chunk_elems;
+  a.tiles_per_chunk = 1;
   a.scale = scale;
   a.write_on_overflow = 0;
   a.zero_fill = 0;
@@ -405,6 +410,15 @@ static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_o
   f.max_norm = max_norm;
   f.ignore_overflow = ignore_overflow;
   return f;
+}
+
+// Write-only passes cut every chunk into tiles so that more, smaller blocks are in flight.
+static void split_for_write(const rg_plan* p, PassArgs& a) {
+  const int64_t tile = p->write_tile_elems;
+  if (tile > 0 && tile < p->chunk_elems && p->n_chunks * ((p->chunk_elems + tile - 1) / tile) <= 0x7fffffffLL) {
+    a.tile_elems = (int32_t)tile;
+    a.tiles_per_chunk = (int32_t)((p->chunk_elems + tile - 1) / tile);
+  }
 }
 
 // Which pointers an operation dereferences.
@@ -449,6 +463,7 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
+  split_for_write(p, a);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, s));
   if (ev) RG_HIP(hipEventRecord(ev[3], s));
   return RG_OK;
@@ -484,7 +499,9 @@ RG_API int rg_scale_cast(rg_plan* p, float scale, void* stream) {
   const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_scale_cast");
   if (rc != RG_OK) return rc;
   DeviceGuard guard(p->device);
-  RG_HIP(launch_pass(kModeWrite, pass_args(p, scale), p->streaming, reinterpret_cast<hipStream_t>(stream)));
+  PassArgs a = pass_args(p, scale);
+  split_for_write(p, a);
+  RG_HIP(launch_pass(kModeWrite, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }
 
@@ -494,6 +511,7 @@ RG_API int rg_zero(rg_plan* p, void* stream) {
   DeviceGuard guard(p->device);
   PassArgs a = pass_args(p, 1.0f);
   a.zero_fill = 1;
+  split_for_write(p, a);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }

@@ -45,8 +45,17 @@ struct StepResult {
 static_assert(sizeof(StepResult) == 32, "result block must stay 32 bytes");
 
 // Tunables (overridable at build time for experiments).
-#ifndef RG_ELEMS_PER_THREAD_ITER
-#define RG_ELEMS_PER_THREAD_ITER 32
+#ifndef RG_REDUCE_ELEMS_PER_THREAD
+#define RG_REDUCE_ELEMS_PER_THREAD 32
+#endif
+#ifndef RG_WRITE_ELEMS_PER_THREAD
+#define RG_WRITE_ELEMS_PER_THREAD 4
+#endif
+#ifndef RG_WRITE_THREADS
+#define RG_WRITE_THREADS 128
+#endif
+#ifndef RG_WRITE_TILE_ELEMS
+#define RG_WRITE_TILE_ELEMS 1024
 #endif
 #ifndef RG_ALIGN_BYTES
 #define RG_ALIGN_BYTES 128
@@ -55,7 +64,13 @@ static_assert(sizeof(StepResult) == 32, "result block must stay 32 bytes");
 #define RG_DEFAULT_CHUNK_ELEMS 16384
 #endif
 constexpr int kBlockThreads = 256;                               // 4 wavefronts of 64
-constexpr int kElemsPerThreadIter = RG_ELEMS_PER_THREAD_ITER;    // elements a thread has in flight per loop iteration
+// Elements a thread has in flight per loop iteration.  Measured on MI355X: a read-only pass
+// is fastest with deep unrolling over 8-16K-element chunks, a pass that also writes with
+// shallow unrolling over small tiles.
+constexpr int kReduceElemsPerThread = RG_REDUCE_ELEMS_PER_THREAD;
+constexpr int kWriteElemsPerThread = RG_WRITE_ELEMS_PER_THREAD;
+constexpr int kWriteThreads = RG_WRITE_THREADS;                  // block size of write-only passes
+constexpr int kWriteTileElems = RG_WRITE_TILE_ELEMS;             // writing passes cut each chunk into tiles of this size
 constexpr unsigned kAlignBytes = RG_ALIGN_BYTES;                 // per-chunk peel of the written (or read-only) side
 constexpr int64_t kChunkQuantum = 2048;    // chunk sizes are multiples of this many elements
 constexpr int64_t kMaxChunkElems = 1 << 20;
@@ -69,6 +84,8 @@ struct PassArgs {
   int32_t* chunk_bad;            // [n_chunks] written when reducing
   const StepResult* result;      // non-null: take coef / overflow gate from the device
   int64_t n_chunks;
+  int32_t tile_elems;            // elements one block handles (== chunk_elems unless the pass splits chunks)
+  int32_t tiles_per_chunk;       // blocks per chunk record
   float scale;
   int32_t write_on_overflow;
   int32_t zero_fill;             // write pass: ignore the sources, store zeros

@@ -34,6 +34,9 @@ typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
 
+// Block size of a pass: write-only passes may use smaller blocks than reducing ones.
+template <int MODE> struct PassThreads { static constexpr int value = (MODE == kModeWrite) ? kWriteThreads : kBlockThreads; };
+
 template <int DT> struct ElemSize { static constexpr int value = 2; };
 template <> struct ElemSize<RG_F32> { static constexpr int value = 4; };
 
@@ -181,12 +184,14 @@ template <> __device__ __forceinline__ bool nonfinite_at<RG_BF16>(const char* p)
 template <int S, int D, int MODE, bool NT>
 __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len, float scale, float coef,
                                               bool raw_copy, float (&acc)[8]) {
+  constexpr int T = PassThreads<MODE>::value;
   constexpr int SS = ElemSize<S>::value;
   constexpr int DS = ElemSize<D>::value;
   constexpr bool kWrite = (MODE & kModeWrite) != 0;
   constexpr bool kReduce = (MODE & kModeReduce) != 0;
   constexpr int E = (SS == 4 || (kWrite && DS == 4)) ? 4 : 8;   // elements per lane per instruction
-  constexpr int U = kElemsPerThreadIter / E;                    // instructions in flight per lane
+  constexpr int kPerThread = kWrite ? kWriteElemsPerThread : kReduceElemsPerThread;
+  constexpr int U = kPerThread >= E ? kPerThread / E : 1;      // instructions in flight per lane
   constexpr int AS = kWrite ? DS : SS;
   const uintptr_t a = kWrite ? reinterpret_cast<uintptr_t>(dp) : reinterpret_cast<uintptr_t>(sp);
   int head = (int)(((kAlignBytes - (unsigned)(a & (kAlignBytes - 1))) & (kAlignBytes - 1)) / (unsigned)AS);
@@ -197,8 +202,8 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
 
   // Unaligned head (< 128 bytes) and ragged tail (< E elements): one element per thread.
   const int nscalar = head + (len - tail0);
-  if (tid < nscalar) {
-    const int i = tid < head ? tid : tail0 + (tid - head);
+  for (int k = tid; k < nscalar; k += T) {
+    const int i = k < head ? k : tail0 + (k - head);
     if (S == D && raw_copy) {
       if (SS == 4) *reinterpret_cast<uint32_t*>(dp + (size_t)i * 4) = *reinterpret_cast<const uint32_t*>(sp + (size_t)i * 4);
       else *reinterpret_cast<unsigned short*>(dp + (size_t)i * 2) = *reinterpret_cast<const unsigned short*>(sp + (size_t)i * 2);
@@ -211,7 +216,7 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
 
   const char* sb = sp + (size_t)head * SS;
   char* db = dp + (size_t)head * DS;
-  constexpr int kIter = kBlockThreads * E * U;   // elements per block iteration
+  constexpr int kIter = T * E * U;   // elements per block iteration
 
   // All U loads of an iteration are issued back to back with no branch between them, so
   // they are all in flight together.  `valid` only guards what is accumulated and stored.
@@ -245,9 +250,9 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   for (; base + kIter <= nbody; base += kIter) {
     Raw<S, E> in[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) in[u] = Mem<S, E, NT>::load(sb + (size_t)(base + (u * kBlockThreads + tid) * E) * SS);
+    for (int u = 0; u < U; ++u) in[u] = Mem<S, E, NT>::load(sb + (size_t)(base + (u * T + tid) * E) * SS);
 #pragma unroll
-    for (int u = 0; u < U; ++u) consume(in[u], base + (u * kBlockThreads + tid) * E, true);
+    for (int u = 0; u < U; ++u) consume(in[u], base + (u * T + tid) * E, true);
   }
   if (base < nbody) {
     // Last, partial iteration: lanes past the end re-read the final vector (an address that
@@ -255,19 +260,19 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
     Raw<S, E> in[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int e = base + (u * kBlockThreads + tid) * E;
+      const int e = base + (u * T + tid) * E;
       in[u] = Mem<S, E, NT>::load(sb + (size_t)(e < nbody ? e : nbody - E) * SS);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int e = base + (u * kBlockThreads + tid) * E;
+      const int e = base + (u * T + tid) * E;
       consume(in[u], e, e < nbody);
     }
   }
 }
 
 // Zero `nbytes` bytes at p (p and nbytes are multiples of 2).
-template <bool NT>
+template <bool NT, int T>
 __device__ __forceinline__ void zero_range(char* p, int nbytes) {
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
   int head = (int)((kAlignBytes - (unsigned)(a & (kAlignBytes - 1))) & (kAlignBytes - 1));
@@ -276,12 +281,12 @@ __device__ __forceinline__ void zero_range(char* p, int nbytes) {
   const int tail0 = head + nvec * 16;
   const int tid = threadIdx.x;
   const int nscalar = (head + (nbytes - tail0)) / 2;
-  if (tid < nscalar) {
-    const int off = tid < head / 2 ? tid * 2 : tail0 + (tid - head / 2) * 2;
+  for (int k = tid; k < nscalar; k += T) {
+    const int off = k < head / 2 ? k * 2 : tail0 + (k - head / 2) * 2;
     *reinterpret_cast<unsigned short*>(p + off) = 0;
   }
   const u32x4 z = {0u, 0u, 0u, 0u};
-  for (int v = tid; v < nvec; v += kBlockThreads) st16<NT>(p + head + (size_t)v * 16, z);
+  for (int v = tid; v < nvec; v += T) st16<NT>(p + head + (size_t)v * 16, z);
 }
 
 template <int S>
@@ -293,8 +298,10 @@ __device__ __forceinline__ int rescan_nonfinite(const char* sp, int len) {
 }
 
 template <int MODE, bool NT>
-__global__ __launch_bounds__(kBlockThreads) void pass_kernel(PassArgs a) {
-  const int64_t c = blockIdx.x;
+__global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs a) {
+  // Block -> (chunk, tile of the chunk).  Reducing passes never split (one partial per chunk).
+  const int64_t c = (MODE & kModeReduce) ? (int64_t)blockIdx.x : (int64_t)(blockIdx.x / (unsigned)a.tiles_per_chunk);
+  const int tile = (MODE & kModeReduce) ? 0 : (int)(blockIdx.x % (unsigned)a.tiles_per_chunk);
   float coef = 1.0f;
   if (a.result != nullptr) {
     // Values produced by the finalize kernel earlier on the same stream.
@@ -303,16 +310,18 @@ __global__ __launch_bounds__(kBlockThreads) void pass_kernel(PassArgs a) {
   }
 
   const ChunkRec rec = a.chunks[c];
-  const int len = rec.len;
-  const char* sp = reinterpret_cast<const char*>(rec.src);
-  char* dp = reinterpret_cast<char*>(rec.dst);
+  const int start = tile * a.tile_elems;
+  if (start >= rec.len && tile > 0) return;
+  const int len = rec.len - start < a.tile_elems ? rec.len - start : a.tile_elems;
+  const char* sp = rec.src ? reinterpret_cast<const char*>(rec.src) + (size_t)start * (rec.src_dtype == RG_F32 ? 4 : 2) : nullptr;
+  char* dp = reinterpret_cast<char*>(rec.dst) + (size_t)start * (rec.dst_dtype == RG_F32 ? 4 : 2);
   const int src_kind = rec.src_dtype;
   const int dst_kind = a.norm_of_source ? rec.src_dtype : rec.dst_dtype;
   const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale == 1.0f;
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (sp == nullptr || a.zero_fill) {
-    if (MODE & kModeWrite) zero_range<NT>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
+    if (MODE & kModeWrite) zero_range<NT, PassThreads<MODE>::value>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
   } else {
     switch (src_kind * 3 + dst_kind) {
       case RG_F32 * 3 + RG_F32: process_chunk<RG_F32, RG_F32, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
@@ -460,7 +469,7 @@ __global__ __launch_bounds__(kBlockThreads) void fill_zero_kernel(char* p, int64
 
 template <int MODE>
 void launch_mode(const PassArgs& a, bool streaming, hipStream_t stream) {
-  const dim3 grid((unsigned)a.n_chunks), block(kBlockThreads);
+  const dim3 grid((unsigned)(a.n_chunks * a.tiles_per_chunk)), block(PassThreads<MODE>::value);
   if (streaming) hipLaunchKernelGGL((pass_kernel<MODE, true>), grid, block, 0, stream, a);
   else hipLaunchKernelGGL((pass_kernel<MODE, false>), grid, block, 0, stream, a);
 }
