@@ -21,8 +21,9 @@ import time
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
 # HBM traffic per launch of the dominant kernel (the write pass), from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs of this same command; see profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+# FETCH_SIZE / WRITE_SIZE runs of this same command, each scaled by what the counter reads for
+# a plain 1 GiB copy (profiles/fused_step_c2_bert_large_hbm_traffic.txt).  Missing = not measured.
+MEASURED_TRAFFIC_BYTES = {"c2_bert_large": 2021538685}
 
 
 def parse_args():
@@ -34,6 +35,9 @@ def parse_args():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--chunk-elems", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 1 GiB fp32 tensor copies first (known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget for the CPU baseline leg")
     return ap.parse_args()
 
@@ -111,6 +115,14 @@ def main() -> int:
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     cfg = step_config(args.workload)
+    if args.calibrate_copy:
+        a = torch.empty(256 << 20, dtype=torch.float32, device=dev).fill_(1.0)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
+        torch.cuda.empty_cache()
     grads, _ = make_grads(cfg, args.seed, device=str(dev))
     n = sum(g.numel() for g in grads)
     ddt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[cfg.bucket_dtype]
