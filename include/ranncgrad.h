@@ -132,6 +132,16 @@ typedef struct rg_step_result {
  * max_norm <= 0 disables clipping (dst = v). */
 int rg_fused_step(rg_plan* plan, float inv_scale, float max_norm, int flags, void* stream);
 
+/* The same step in two calls, for callers that must look at the overflow flag in between
+ * (the amp context exit updates the loss scale before the user asks for clipping:
+ * pyrannc/amp/__init__.py:44-65 runs at scale_loss exit, RaNNCModule.clip_grad_norm later).
+ * rg_step_begin  = pass 1 + norm/flag (result.coef = 1, clipped = 0);
+ * rg_step_finish = clip decision for max_norm from the sums pass 1 left on the device, then
+ *                  pass 2 with the inv_scale given to rg_step_begin.
+ * Together they move exactly the bytes of rg_fused_step. */
+int rg_step_begin(rg_plan* plan, float inv_scale, void* stream);
+int rg_step_finish(rg_plan* plan, float max_norm, int flags, void* stream);
+
 /* One pass: dst = round_dst(float(x) * inv_scale), overflow flag and norm as above, no
  * clip.  Apex multi_tensor_scale semantics (LossScaler.unscale). */
 int rg_unscale_pack(rg_plan* plan, float inv_scale, void* stream);
@@ -147,6 +157,13 @@ int rg_grad_norm(rg_plan* plan, void* stream);
  * src/comp/DistributedGradLocator.cpp:59, DistributedParamLocatorBase.cpp:130-131,
  * and Apex's master<->model copies. */
 int rg_scale_cast(rg_plan* plan, float scale, void* stream);
+
+/* The same for ONE tensor, without a plan and without any allocation (src_dev == NULL
+ * stores zeros): the one-off copies of DistributedParamLocator::store / set / setScalarType
+ * (src/comp/DistributedParamLocator.cpp:14-83) and of gather's padded send buffer
+ * (src/comp/DistributedParamLocatorBase.cpp:124-131). */
+int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t numel, int src_dtype, int dst_dtype,
+                         float scale, int device, void* stream);
 
 /* dst = 0 for every tensor.  ParamStorage::clearParamGrads, src/comp/ParamStorage.cpp:540-557. */
 int rg_zero(rg_plan* plan, void* stream);

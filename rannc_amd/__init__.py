@@ -1,0 +1,175 @@
+"""rannc_amd: the per-step parameter/gradient path of RaNNC on one MI355X.
+
+``RaNNCModule`` keeps the constructor arguments and the hot-path methods of
+``pyrannc.RaNNCModule`` (``pyrannc/__init__.py:206-593``): ``clip_grad_norm``,
+``_calc_grad_norm``, ``zero_grad``, ``get_param``, the ZeRO segment accessors and the
+optimizer patching.  The wrapped model runs as it is, on one GPU: tracing, profiling,
+partitioning and pipelining are not part of this package.  All arithmetic on parameters and
+gradients goes through ``libranncgrad`` (hand-written HIP for gfx950); there is no CPU or
+PyTorch fallback for it.
+"""
+from __future__ import annotations
+
+import logging
+
+import torch
+
+from . import _pyrannc
+from .dist_param import (DistributeModelParams, get_dist_param_range, get_dist_param_segment,  # noqa: F401
+                         load_dist_param, remove_dist_param, set_dist_param, set_dist_param_dtype,
+                         store_dist_param)
+from .opt import patch_optimizer
+
+logger = logging.getLogger("rannc")
+
+
+def get_rank() -> int:
+    return _pyrannc.get_rank()
+
+
+def get_world_size() -> int:
+    return _pyrannc.get_world_size()
+
+
+def barrier() -> None:
+    _pyrannc.barrier()
+
+
+def clear() -> None:
+    _pyrannc.clear()
+
+
+class RaNNCModule(_pyrannc.RaNNCModule):
+    r"""
+    Wraps a ``torch.nn.Module`` (``pyrannc/__init__.py:206-252``).
+
+    :param model: Model to wrap.
+    :param optimizer: Optimizer; it is patched so that it steps on the parameters this
+        process owns (``patch_optimizer``).
+    :param enable_apex_amp: Master parameters and gradients are fp32 (amp O2).
+    :param allreduce_amp_master_params: Gradients are reduced in fp32.
+    :param enable_zero: ZeRO-style sharding of master parameters / optimizer state
+        (requires ``enable_apex_amp``).
+    :param consolidate_grads: keep gradients in per-dtype flat buckets (the reference's
+        ``consolidate_grads`` configuration item, ``src/Config.cpp:32,146``).
+    """
+
+    def __init__(self, model, optimizer=None, gather_inputs=True, enable_apex_amp=False,
+                 allreduce_amp_master_params=False, enable_zero=False, check_unused_values=True,
+                 offload_params=False, consolidate_grads=False):
+        if enable_zero and not enable_apex_amp:                      # pyrannc/__init__.py:224-225
+            raise ValueError("enable_zero requires enable_apex_amp")
+        super().__init__(enable_apex_amp, allreduce_amp_master_params, enable_zero, check_unused_values,
+                         offload_params)
+        self.model = model
+        self.optimizer = optimizer
+        self.gather_inputs = gather_inputs
+        self.enable_apex_amp = enable_apex_amp
+        self.allreduce_amp_master_params = allreduce_amp_master_params
+        self.enable_zero = enable_zero
+        self.offload_params = offload_params
+        self.consolidate_grads = consolidate_grads
+        self.amp_master_param_registered = False
+        self.ready = False
+        self.used_param_ids = set()
+        self.name_to_param = {}
+        self.name_to_pid = {}
+        self.device = torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() \
+            else torch.device("cpu")
+
+    # ------------------------------------------------------------------ deployment
+    def _deploy(self) -> None:
+        if self.device.type != "cuda":
+            raise RuntimeError("rannc_amd needs a GPU: parameters and gradients are processed by HIP kernels only")
+        named = dict(self.model.named_parameters())
+        for n, p in named.items():
+            if not p.is_cuda:
+                raise ValueError(f"parameter {n} is on {p.device}; move the model to the GPU first")
+        self.name_to_param = named
+        ids = self.init(named, consolidate_grads=self.consolidate_grads)
+        self.name_to_pid = ids
+        self.used_param_ids = set(ids.values())
+        if self.enable_zero:                                          # pyrannc/__init__.py:289-290
+            self.align_params()
+        if self.optimizer is not None:
+            patch_optimizer(self, self.optimizer)
+        self.ready = True
+
+    def __call__(self, *args, **kwargs):
+        if not self.ready:
+            self._deploy()
+        if self.enable_zero:
+            self.sync_param_zero(False)                               # GraphLauncher.cpp:366-368
+        self.prepare_backward()                                       # GraphLauncher.cpp:468
+        return self.model(*args, **kwargs)
+
+    def parameters(self, *args, **kwargs):
+        return self.model.parameters(*args, **kwargs)
+
+    def named_parameters(self, *args, **kwargs):
+        return self.model.named_parameters(*args, **kwargs)
+
+    # ------------------------------------------------------------------ per-step API
+    def _setup_amp_params(self):
+        if not self.amp_master_param_registered:                      # pyrannc/__init__.py:374-379
+            from .amp import patch_amp_scaler, register_amp_params
+            register_amp_params(self.optimizer)
+            patch_amp_scaler()
+            self.amp_master_param_registered = True
+
+    def clip_grad_norm(self, max_grad_norm):
+        r"""
+        Clips gradients by their global L2 norm (``pyrannc/__init__.py:381-394``): iff
+        ``norm + 1e-6 > max_grad_norm`` every gradient is multiplied by
+        ``max_grad_norm / (norm + 1e-6)``.  With amp in fused mode the pending unscale is
+        completed and clipped in the same pass over the gradients.
+        """
+        if not self.ready:
+            self._deploy()
+        if self.enable_apex_amp:
+            self._setup_amp_params()
+            stash = getattr(self.optimizer, "_amp_stash", None)
+            if stash is not None and stash.pending_finish and not stash.all_fp32_from_fp32_params:
+                from .amp import finish_unscale
+                finish_unscale(self.optimizer, float(torch.tensor(max_grad_norm, dtype=torch.float32)))
+                return
+            if stash is not None and stash.pending_finish:
+                from .amp import finish_unscale
+                finish_unscale(self.optimizer)
+        super().clip_grad_norm(max_grad_norm)
+
+    def _calc_grad_norm(self):
+        if not self.ready:
+            self._deploy()
+        if self.enable_apex_amp:
+            self._setup_amp_params()
+            stash = getattr(self.optimizer, "_amp_stash", None)
+            if stash is not None and stash.pending_finish:
+                from .amp import finish_unscale
+                finish_unscale(self.optimizer)
+        return super().calc_grad_norm()
+
+    def zero_grad(self):
+        r"""Sets zeros to gradients of model parameters (``pyrannc/__init__.py:453-457``)."""
+        if not self.ready:
+            self._deploy()
+        super().zero_grad()
+
+    def get_param(self, name, amp_master_param=False):
+        if name not in self.name_to_pid:
+            raise RuntimeError(f"Parameter not found: {name}")       # pyrannc/__init__.py:466-467
+        return super().get_param(self.name_to_pid[name], amp_master_param)
+
+    def get_param_grad(self, name, amp_master_param=False):
+        p = self.get_param(name, amp_master_param)
+        return p.grad
+
+    @property
+    def use_amp_master_params_flag(self):
+        return self.use_amp_master_params()
+
+    def __del__(self):
+        try:
+            self.undeploy()
+        except Exception:
+            pass

@@ -44,9 +44,12 @@ SIGNATURES = {
     "rg_plan_total_numel": (_i64, [_vp]),
     "rg_plan_set_streaming": (_i, [_vp, _i]),
     "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
+    "rg_step_begin": (_i, [_vp, _f, _vp]),
+    "rg_step_finish": (_i, [_vp, _f, _i, _vp]),
     "rg_unscale_pack": (_i, [_vp, _f, _vp]),
     "rg_grad_norm": (_i, [_vp, _vp]),
     "rg_scale_cast": (_i, [_vp, _f, _vp]),
+    "rg_scale_cast_single": (_i, [_vp, _vp, _i64, _i, _i, _f, _i, _vp]),
     "rg_zero": (_i, [_vp, _vp]),
     "rg_fill_zero": (_i, [_vp, _i64, _i, _vp]),
     "rg_result_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
@@ -181,6 +184,12 @@ class Plan:
     def fused_step(self, inv_scale: float, max_norm: float, flags: int = RG_STEP_DEFAULT, stream: int = 0) -> None:
         check(lib.rg_fused_step(self._handle, inv_scale, max_norm, flags, _vp(stream)))
 
+    def step_begin(self, inv_scale: float, stream: int = 0) -> None:
+        check(lib.rg_step_begin(self._handle, inv_scale, _vp(stream)))
+
+    def step_finish(self, max_norm: float, flags: int = RG_STEP_DEFAULT, stream: int = 0) -> None:
+        check(lib.rg_step_finish(self._handle, max_norm, flags, _vp(stream)))
+
     def unscale_pack(self, inv_scale: float, stream: int = 0) -> None:
         check(lib.rg_unscale_pack(self._handle, inv_scale, _vp(stream)))
 
@@ -217,6 +226,12 @@ class Plan:
         out = _vp()
         check(lib.rg_result_device_ptr(self._handle, C.byref(out)))
         return int(out.value)
+
+
+def scale_cast_single(src_ptr: Optional[int], dst_ptr: int, numel: int, src_dtype: int, dst_dtype: int,
+                      scale: float, device: int, stream: int = 0) -> None:
+    check(lib.rg_scale_cast_single(_vp(src_ptr or None), _vp(dst_ptr or None), numel, src_dtype, dst_dtype,
+                                   scale, device, _vp(stream)))
 
 
 def fill_zero(ptr: int, nbytes: int, device: int, stream: int = 0) -> None:

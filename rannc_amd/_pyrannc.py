@@ -1,0 +1,211 @@
+"""The entry points of the reference's extension module ``pyrannc._pyrannc``
+(``src/main.cpp:30-522``) that the per-step parameter/gradient path uses, with the same
+names, argument meaning and error behaviour, for one process on one GPU.
+
+Everything that only exists to trace, partition or pipeline a model is absent.
+Unknown ids raise ``ValueError`` (the reference's ``std::invalid_argument``); library
+failures raise ``RuntimeError``.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from .dist_param_locator import DistributedParamLocator
+from .param_storage import ParamStorage
+
+_param_storage = ParamStorage()
+_dist_param_locator = DistributedParamLocator()
+_tracing_state = True
+
+
+def get_param_storage() -> ParamStorage:
+    return _param_storage
+
+
+def get_dist_param_locator() -> DistributedParamLocator:
+    return _dist_param_locator
+
+
+# -- process state (src/main.cpp:55-59); one process, one GPU
+def get_rank() -> int:
+    return 0
+
+
+def get_world_size() -> int:
+    return 1
+
+
+def barrier() -> None:
+    return None
+
+
+def clear() -> None:
+    global _param_storage
+    for gid in list(_param_storage.graph_params):
+        _param_storage.undeploy(gid)
+    _param_storage = ParamStorage()
+    _dist_param_locator.clear()
+
+
+def set_tracing_state(enable: bool) -> None:
+    global _tracing_state
+    _tracing_state = bool(enable)
+
+
+# -- tensor collectives (src/main.cpp:78-136).  With one rank a sum or a min over ranks,
+# -- a broadcast and an all-gather return their input.
+def allreduce_tensor(tensor: torch.Tensor, sum: bool) -> None:   # noqa: A002 - the reference's name
+    if not isinstance(tensor, torch.Tensor):
+        raise ValueError("allreduce_tensor expects a tensor")
+
+
+def bcast_tensor(tensor: torch.Tensor, root: int) -> torch.Tensor:
+    if root != 0:
+        raise ValueError(f"root {root} is not a rank of this world (size 1)")
+    return tensor.cuda()
+
+
+def all_gather(ten: torch.Tensor, buf: torch.Tensor) -> None:
+    if buf.numel() != ten.numel():
+        raise ValueError("all_gather: receive buffer must hold world_size * numel elements")
+    from .multi_tensor import copy_cast_
+    with torch.no_grad():
+        copy_cast_(buf.view(-1), ten.contiguous().view(-1))
+
+
+# -- amp masters (src/main.cpp:191-200)
+def register_amp_master_param(model_param_id: int, param: torch.Tensor) -> None:
+    _param_storage.register_amp_master_param(model_param_id, id(param), param)
+
+
+# -- distributed parameters (src/main.cpp:202-245)
+def store_dist_param(param: torch.Tensor) -> torch.Tensor:
+    return _dist_param_locator.store(id(param), param)
+
+
+def load_dist_param(pid: int) -> torch.Tensor:
+    return _dist_param_locator.load(pid)
+
+
+def set_dist_param(pid: int, param: torch.Tensor) -> None:
+    _dist_param_locator.set(pid, param)
+
+
+def get_dist_param_segment(pid: int) -> torch.Tensor:
+    return _dist_param_locator.get_segment(pid)
+
+
+def set_dist_param_dtype(pid: int, dtype: torch.dtype) -> None:
+    _dist_param_locator.set_scalar_type(pid, dtype)
+
+
+def get_dist_param_range(pid: int) -> Tuple[int, int]:
+    return _dist_param_locator.get_segment_range(pid)
+
+
+def remove_dist_param(pid: int) -> None:
+    _dist_param_locator.remove(pid)
+
+
+def dist_param_registered(pid: int) -> bool:
+    return _dist_param_locator.registered(pid)
+
+
+def get_param_ranks(pid: int):
+    _param_storage.get_param_tensor(pid)
+    return {0}
+
+
+class RaNNCModule:
+    """The methods of the bound C++ ``RaNNCModule`` (``src/main.cpp:257-450``) that sit on the
+    per-step path.  ``init`` here only registers the parameters of the (whole, unpartitioned)
+    model under one graph id; there is no tracing, profiling or partitioning."""
+
+    _next_id = 0
+
+    def __init__(self, use_amp_master_params: bool = False, allreduce_amp_master_params: bool = False,
+                 enable_zero: bool = False, check_unused_values: bool = True, offload_params: bool = False):
+        self._use_amp_master_params = bool(use_amp_master_params)
+        self._allreduce_amp_master_params = bool(allreduce_amp_master_params)
+        self._enable_zero = bool(enable_zero)
+        self.graph_id = f"graph_{RaNNCModule._next_id}"
+        RaNNCModule._next_id += 1
+        self._deployed = False
+
+    def init(self, named_params: Dict[str, torch.Tensor], consolidate_grads: bool = False) -> Dict[str, int]:
+        """Register ``name -> parameter`` and deploy them; returns ``name -> id``
+        (``RaNNCModule::init`` returns the used-parameter ids, ``src/comp/RaNNCModule.cpp:160-501``)."""
+        ids = {}
+        for name, p in named_params.items():
+            _param_storage.register_param(id(p), p)
+            ids[name] = id(p)
+        _param_storage.deploy(self.graph_id, ids, enable_zero=self._enable_zero, consolidate=consolidate_grads,
+                              use_amp_master_params=self._use_amp_master_params,
+                              allreduce_amp_master_params=self._allreduce_amp_master_params)
+        self._deployed = True
+        return ids
+
+    def _check(self) -> None:
+        if not self._deployed:
+            raise RuntimeError("RaNNCModule is not initialised")
+
+    def prepare_backward(self) -> None:
+        self._check()
+        _param_storage.prepare_backward(self.graph_id)
+
+    def allreduce_grads(self) -> None:
+        self._check()
+        _param_storage.allreduce_param_grads(self.graph_id)
+
+    def allreduce_grads_zero(self) -> None:
+        self._check()
+        self._staging = _param_storage.allreduce_param_grads_zero(self.graph_id)
+
+    def clip_grad_norm(self, max_grad_norm: float) -> None:
+        self._check()
+        _param_storage.clip_grad_norm(self.graph_id, float(torch.tensor(max_grad_norm, dtype=torch.float32)),
+                                      self._use_amp_master_params)
+
+    def calc_grad_norm(self) -> float:
+        self._check()
+        return _param_storage.calc_grad_global_l2_norm(self.graph_id, self._use_amp_master_params)
+
+    def zero_grad(self) -> None:
+        self._check()
+        _param_storage.clear_param_grads(self.graph_id)
+
+    def use_amp_master_params(self) -> bool:
+        return self._use_amp_master_params
+
+    def align_params(self) -> None:
+        self._check()
+        _param_storage.align_buffer_zero(self.graph_id)
+
+    def sync_param_zero(self, grad: bool) -> None:
+        self._check()
+        _param_storage.bcast_params_zero(self.graph_id, grad)
+
+    def set_grad_to_local_param_segment(self) -> None:
+        self._check()
+        _param_storage.set_grad_to_local_param_segment(self.graph_id)
+
+    def get_local_param_range(self, param_id: int) -> Tuple[int, int]:
+        self._check()
+        return _param_storage.get_local_param_range(self.graph_id, param_id)
+
+    def get_local_param_segment(self, param_id: int) -> torch.Tensor:
+        self._check()
+        return _param_storage.get_local_param_segment(self.graph_id, param_id)
+
+    def get_param(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
+        self._check()
+        if amp_master_param and _param_storage.has_amp_master_param(param_id):
+            return _param_storage.get_amp_master_param_tensor(param_id)
+        return _param_storage.get_param_tensor(param_id)
+
+    def undeploy(self) -> None:
+        if self._deployed:
+            _param_storage.undeploy(self.graph_id)
+            self._deployed = False

@@ -1,0 +1,335 @@
+"""Mixed-precision support of the per-step path.
+
+Two layers live here:
+
+* the functions of ``pyrannc/amp/__init__.py`` with their signatures and behaviour:
+  ``register_amp_params`` (``:13-18``), ``named_master_params`` (``:21-41``),
+  ``patch_amp_scaler`` (``:44-65``), ``unset_master_grads`` (``:68-70``);
+* the part of NVIDIA Apex amp (O2) those functions lean on, which is not in the reference
+  tree (``docker/ubuntu/runtime/Dockerfile:13`` pins an external commit): fp32 master
+  parameters, ``scale_loss``, a ``LossScaler`` whose ``unscale`` is the fused HIP kernel
+  (Apex's ``multi_tensor_scale``: ``master_grad = float(model_grad) * (1 / scale)`` plus an
+  inf/NaN flag), the skip of ``optimizer.step`` after an overflow and the master -> model
+  copy after a step.  Attribute names follow Apex (``_amp_state.loss_scalers``,
+  ``optimizer._amp_stash.all_fp16_params`` ...) because the reference reads them.
+
+The dynamic loss-scale schedule (halve on overflow, double after ``scale_window`` clean
+steps) is this project's own statement of the usual policy; Apex's is not in the tree.
+
+Gradient accumulation over several ``scale_loss`` contexts is not supported: master
+gradients are overwritten, not accumulated, by each unscale.
+"""
+from __future__ import annotations
+
+import contextlib
+from typing import Iterator, List, Optional, Tuple
+
+import torch
+
+from .. import _lib, _pyrannc
+from ..multi_tensor import TensorPlan
+from ..tensor_coll import _allreduce_min, _allreduce_sum
+
+
+class _AmpState:
+    def __init__(self) -> None:
+        self.loss_scalers: List["LossScaler"] = []
+        self.opt_level: Optional[str] = None
+
+
+_amp_state = _AmpState()
+
+
+class _AmpStash:
+    """The lists Apex hangs on ``optimizer._amp_stash`` (read at ``pyrannc/amp/__init__.py:9-11``)."""
+
+    def __init__(self) -> None:
+        self.all_fp16_params: List[torch.Tensor] = []
+        self.all_fp32_from_fp16_params: List[torch.Tensor] = []
+        self.all_fp32_from_fp32_params: List[torch.Tensor] = []
+        self.already_patched = False
+        self.unscale_plan: Optional[TensorPlan] = None
+        self.unscale_key: Optional[tuple] = None
+        self.copy_back_plan: Optional[TensorPlan] = None
+        self.pending_finish = False        # fused mode: the write pass has not run yet
+        self.fused = False
+        self.last_result = None            # rg_step_result of the last unscale
+        self.norm_is_fresh = False
+        # packed fp32 bucket the master gradients are views of (the reference's
+        # consolidated_master_grads_, src/comp/ParamStorage.cpp:68-70, 92-97): stable
+        # addresses, so the device table is built once
+        self.master_grad_bucket: Optional[torch.Tensor] = None
+        self.master_grad_views: List[torch.Tensor] = []
+
+
+class LossScaler:
+    """Loss scale with the fused unscale + overflow check."""
+
+    def __init__(self, loss_scale="dynamic", init_scale: float = 2.0 ** 16, scale_factor: float = 2.0,
+                 scale_window: int = 2000, min_loss_scale: Optional[float] = None,
+                 max_loss_scale: float = 2.0 ** 24) -> None:
+        self.dynamic = loss_scale == "dynamic"
+        self._loss_scale = min(max_loss_scale, init_scale) if self.dynamic else float(loss_scale)
+        self._scale_seq_len = scale_window
+        self._scale_factor = scale_factor
+        self._min_loss_scale = min_loss_scale
+        self._max_loss_scale = max_loss_scale
+        self._unskipped = 0
+        self._has_overflow = False
+
+    def loss_scale(self) -> float:
+        return self._loss_scale
+
+    def clear_overflow_state(self) -> None:
+        self._has_overflow = False
+
+    def unscale(self, stash: _AmpStash, model_grads: List[torch.Tensor], master_grads: List[torch.Tensor]) -> None:
+        """``master_grad = float(model_grad) * (1 / scale)`` for every pair in one launch, with the
+        inf/NaN flag and - for free - the gradient norm.  In fused mode only the read pass runs
+        here; the values are written by ``finish_unscale``."""
+        key = tuple((g.data_ptr(), g.numel(), g.dtype, m.data_ptr(), m.dtype) for g, m in zip(model_grads, master_grads))
+        if stash.unscale_plan is None or stash.unscale_key != key:
+            if stash.unscale_plan is not None:
+                stash.unscale_plan.close()
+            stash.unscale_plan = TensorPlan(model_grads, master_grads)
+            stash.unscale_key = key
+        inv = 1.0 / self._loss_scale
+        with torch.no_grad():
+            if stash.fused:
+                stash.unscale_plan.step_begin(inv)
+                stash.pending_finish = True
+            else:
+                stash.unscale_plan.unscale_pack(inv)
+        stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
+        stash.norm_is_fresh = True
+        if stash.last_result.overflow:
+            self._has_overflow = True
+
+    def update_scale(self) -> bool:
+        """Returns True when the step must be skipped.  Own schedule (see module docstring)."""
+        if self._has_overflow and self.dynamic:
+            should_skip = True
+            self._loss_scale = self._loss_scale / 2.0
+            if self._min_loss_scale:
+                self._loss_scale = max(self._min_loss_scale, self._loss_scale)
+            self._unskipped = 0
+        else:
+            should_skip = False
+            self._unskipped += 1
+        if self._unskipped == self._scale_seq_len and self.dynamic:
+            self._loss_scale = min(self._max_loss_scale, self._loss_scale * self._scale_factor)
+            self._unskipped = 0
+        return should_skip
+
+
+def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_level: str = "O2",
+               loss_scale="dynamic", max_loss_scale: float = 2.0 ** 24, min_loss_scale: Optional[float] = None,
+               half_dtype: torch.dtype = torch.float16, fused: bool = False
+               ) -> Tuple[torch.nn.Module, torch.optim.Optimizer]:
+    """O2-style set-up: the model's floating-point parameters (batch-norm layers excepted)
+    become ``half_dtype``; the optimizer is re-pointed at fp32 masters created as
+    ``param.detach().clone().float()``; ``optimizer.step`` is wrapped to skip once after an
+    overflow and to copy masters back into the model afterwards.
+
+    ``fused=True`` defers the write of the unscaled master gradients from the ``scale_loss``
+    exit to the next ``clip_grad_norm`` / ``optimizer.step``, so that unscale, norm, clip and
+    pack move ``(2s + d)`` bytes per element; until then master ``.grad`` holds stale data."""
+    if opt_level != "O2":
+        raise ValueError("only opt_level='O2' (fp32 masters for half parameters) is provided")
+    bn = torch.nn.modules.batchnorm._BatchNorm
+    for mod in model.modules():
+        if isinstance(mod, bn):
+            continue
+        for p in mod.parameters(recurse=False):
+            if p.dtype == torch.float32:
+                p.data = p.data.to(half_dtype)
+        for name, b in mod.named_buffers(recurse=False):
+            if b.dtype == torch.float32:
+                mod._buffers[name] = b.to(half_dtype)
+    stash = _AmpStash()
+    stash.fused = fused
+    for group in optimizer.param_groups:
+        new_params = []
+        for p in group["params"]:
+            if p.dtype in (torch.float16, torch.bfloat16):
+                master = p.detach().clone().float()
+                master.requires_grad_(p.requires_grad)
+                stash.all_fp16_params.append(p)
+                stash.all_fp32_from_fp16_params.append(master)
+                if p in optimizer.state:
+                    optimizer.state[master] = optimizer.state.pop(p)
+                new_params.append(master)
+            else:
+                stash.all_fp32_from_fp32_params.append(p)
+                new_params.append(p)
+        group["params"] = new_params
+    optimizer._amp_stash = stash
+    scaler = LossScaler(loss_scale, min_loss_scale=min_loss_scale, max_loss_scale=max_loss_scale)
+    _amp_state.loss_scalers = [scaler]
+    _amp_state.opt_level = opt_level
+    _patch_step(optimizer)
+    return model, optimizer
+
+
+def master_params(optimizer: torch.optim.Optimizer) -> Iterator[torch.Tensor]:
+    """``apex.amp.master_params``: every parameter the optimizer steps on."""
+    for group in optimizer.param_groups:
+        for p in group["params"]:
+            yield p
+
+
+def finish_unscale(optimizer: torch.optim.Optimizer, max_norm: float = 0.0) -> None:
+    """Fused mode: run the deferred write pass (clip to ``max_norm`` when > 0)."""
+    stash = optimizer._amp_stash
+    if stash.pending_finish:
+        with torch.no_grad():
+            stash.unscale_plan.step_finish(float(max_norm))
+        stash.pending_finish = False
+        stash.norm_is_fresh = False
+
+
+def _master_to_model(optimizer: torch.optim.Optimizer) -> None:
+    """Apex's post-step copy (``multi_tensor_scale`` with scale 1): ``model = half(master)``,
+    round to nearest even, one launch for all pairs."""
+    stash = optimizer._amp_stash
+    if not stash.all_fp16_params:
+        return
+    if stash.copy_back_plan is None:
+        stash.copy_back_plan = TensorPlan([m.detach() for m in stash.all_fp32_from_fp16_params],
+                                          [p.detach() for p in stash.all_fp16_params])
+    with torch.no_grad():
+        stash.copy_back_plan.scale_cast(1.0)
+
+
+def _patch_step(optimizer: torch.optim.Optimizer) -> None:
+    stash = optimizer._amp_stash
+    if stash.already_patched:
+        return
+    old_step = optimizer.step
+
+    def new_step(*args, **kwargs):
+        if getattr(stash, "skip_next_step", False):
+            stash.skip_next_step = False
+            stash.pending_finish = False
+            return None
+        finish_unscale(optimizer)
+        ret = old_step(*args, **kwargs)
+        _master_to_model(optimizer)
+        stash.norm_is_fresh = False
+        return ret
+
+    optimizer.step = new_step
+    stash.already_patched = True
+
+
+@contextlib.contextmanager
+def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
+    """``with amp.scale_loss(loss, optimizer) as scaled_loss: scaled_loss.backward()``.
+    On exit: unscale the model gradients into the master gradients (fused kernel), update the
+    loss scale, and arm a one-shot skip of ``optimizer.step`` after an overflow."""
+    scaler = _amp_state.loss_scalers[0]
+    stash = optimizer._amp_stash
+    yield loss.float() * scaler.loss_scale()
+    model_grads, master_grads = [], []
+    if stash.master_grad_bucket is None and stash.all_fp32_from_fp16_params:
+        masters = stash.all_fp32_from_fp16_params
+        offs, lens = _lib.bucket_layout([m.numel() for m in masters], [_lib.RG_F32] * len(masters))
+        stash.master_grad_bucket = torch.empty(lens[_lib.RG_F32], dtype=torch.float32, device=masters[0].device)
+        stash.master_grad_views = [stash.master_grad_bucket.narrow(0, o, m.numel()).view(m.shape)
+                                   for o, m in zip(offs, masters)]
+    for i, (p, m) in enumerate(zip(stash.all_fp16_params, stash.all_fp32_from_fp16_params)):
+        if p.grad is None:
+            continue
+        if m.grad is None:
+            m.grad = stash.master_grad_views[i]
+        model_grads.append(p.grad)
+        master_grads.append(m.grad)
+    scaler.clear_overflow_state()
+    if model_grads:
+        scaler.unscale(stash, model_grads, master_grads)
+    # fp32 parameters keep their own .grad; it carries the loss scale too
+    fp32_grads = [p.grad for p in stash.all_fp32_from_fp32_params if p.grad is not None]
+    if fp32_grads:
+        plan = TensorPlan(fp32_grads, fp32_grads)
+        with torch.no_grad():
+            plan.unscale_pack(1.0 / scaler.loss_scale())
+        if plan.result().overflow:
+            scaler._has_overflow = True
+        plan.close()
+    should_skip = scaler.update_scale()
+    if should_skip:
+        stash.skip_next_step = True
+    for p in stash.all_fp16_params:       # Apex O2 drops the half grads once they are unscaled
+        p.grad = None
+
+
+# --------------------------------------------------------------------------- reference API
+
+def zip_params(optimizer):
+    stash = optimizer._amp_stash
+    return zip(stash.all_fp32_from_fp16_params, stash.all_fp16_params)
+
+
+def register_amp_params(optimizer):
+    """``pyrannc/amp/__init__.py:13-18``."""
+    for master_p, model_p in zip_params(optimizer):
+        if model_p in getattr(optimizer, "param_zero_segment_to_id", {}):
+            _pyrannc.register_amp_master_param(optimizer.param_zero_segment_to_id[model_p], master_p)
+        else:
+            _pyrannc.register_amp_master_param(id(model_p), master_p)
+
+
+def named_master_params(model, optimizer, zero=False):
+    """``pyrannc/amp/__init__.py:21-41``."""
+    if hasattr(optimizer._amp_stash, "all_fp32_from_fp16_params"):
+        amp_param_map = {model_p: master_p for master_p, model_p in zip_params(optimizer)}
+        if zero:
+            pid_to_name = {pid: n for n, pid in model.name_to_pid.items()}
+            pid_to_segment = {pid: segment for segment, pid in optimizer.param_zero_segment_to_id.items()}
+            for pid, segment in pid_to_segment.items():
+                if segment.dtype == torch.float:
+                    amp_param_map[segment] = segment
+            for model_p, master_p in amp_param_map.items():
+                yield pid_to_name[optimizer.param_zero_segment_to_id[model_p]], master_p
+        else:
+            for p in model.parameters():
+                if p.dtype == torch.float:
+                    amp_param_map[p] = p
+            for n, p in model.named_parameters():
+                yield n, amp_param_map[p]
+
+
+def patch_amp_scaler():
+    """``pyrannc/amp/__init__.py:44-65``: after the scaler's own ``update_scale`` share the
+    overflow flag (sum over ranks) and, on overflow anywhere, adopt the smallest loss scale."""
+    scaler = _amp_state.loss_scalers[0]
+    if getattr(scaler, "_rannc_patched", False):
+        return
+
+    def decorate(func):
+        def wrapper():
+            had_overflow = func()
+
+            # Share if overflow happens on any of ranks
+            flag_overflow = torch.IntTensor([0]).cuda()
+            if had_overflow:
+                flag_overflow = torch.IntTensor([1]).cuda()
+            _allreduce_sum(flag_overflow)
+
+            if flag_overflow.item() > 0:
+                scale_buf = torch.IntTensor([int(scaler._loss_scale)]).cuda()
+                _allreduce_min(scale_buf)
+                scaler._loss_scale = scale_buf.item()
+                scaler._unskipped = 0
+                return True
+            return False
+        return wrapper
+
+    scaler.update_scale = decorate(scaler.update_scale)
+    scaler._rannc_patched = True
+
+
+def unset_master_grads(optimizer):
+    """``pyrannc/amp/__init__.py:68-70``."""
+    for p in master_params(optimizer):
+        p.grad = None

@@ -71,6 +71,7 @@ struct rg_plan {
   int64_t n_chunks = 0;
   bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
   int64_t write_tile_elems = kWriteTileElems;
+  float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
   std::vector<TensorDesc> host_tensors;
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
 
@@ -383,6 +384,7 @@ RG_API int rg_plan_set_streaming(rg_plan* p, int mode) {
 
 static PassArgs pass_args(const rg_plan* p, float scale) {
   PassArgs a;
+  memset(&a, 0, sizeof(a));
   a.chunks = p->d_chunks;
   a.chunk_sumsq = p->d_chunk_sumsq;
   a.chunk_bad = p->d_chunk_bad;
@@ -469,6 +471,40 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   return RG_OK;
 }
 
+RG_API int rg_step_begin(rg_plan* p, float inv_scale, void* stream) {
+  const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_step_begin");
+  if (rc != RG_OK) return rc;
+  if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
+    set_error("rg_step_begin: inv_scale must be a non-zero number");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  RG_HIP(launch_pass(kModeReduce, pass_args(p, inv_scale), p->streaming, s));
+  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
+  p->begun_inv_scale = inv_scale;
+  return RG_OK;
+}
+
+RG_API int rg_step_finish(rg_plan* p, float max_norm, int flags, void* stream) {
+  const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_step_finish");
+  if (rc != RG_OK) return rc;
+  if (p->begun_inv_scale == 0.0f) {
+    set_error("rg_step_finish: no rg_step_begin is pending on this plan");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  RG_HIP(launch_finalize_total(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
+  PassArgs a = pass_args(p, p->begun_inv_scale);
+  a.result = p->d_result;
+  a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
+  split_for_write(p, a);
+  RG_HIP(launch_pass(kModeWrite, a, p->streaming, s));
+  p->begun_inv_scale = 0.0f;
+  return RG_OK;
+}
+
 RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_unscale_pack");
   if (rc != RG_OK) return rc;
@@ -502,6 +538,47 @@ RG_API int rg_scale_cast(rg_plan* p, float scale, void* stream) {
   PassArgs a = pass_args(p, scale);
   split_for_write(p, a);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
+  return RG_OK;
+}
+
+RG_API int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t numel, int src_dtype, int dst_dtype,
+                                float scale, int device, void* stream) {
+  const int ss = elem_size(src_dtype), ds = elem_size(dst_dtype);
+  if (ss < 0 || ds < 0 || numel < 0 || (numel > 0 && dst_dev == nullptr)) {
+    set_error("rg_scale_cast_single: bad arguments (dtypes %d->%d, numel %lld)", src_dtype, dst_dtype, (long long)numel);
+    return RG_EINVAL;
+  }
+  int rc = check_pointer(src_dev, ss, "src", 0);
+  if (rc == RG_OK) rc = check_pointer(dst_dev, ds, "dst", 0);
+  if (rc != RG_OK) return rc;
+  if (src_dev == dst_dev && src_dtype != dst_dtype) {
+    set_error("rg_scale_cast_single: in place but changes dtype");
+    return RG_EINVAL;
+  }
+  if (numel == 0) return RG_OK;
+  const int64_t chunk = RG_DEFAULT_CHUNK_ELEMS;
+  const int64_t n_chunks = (numel + chunk - 1) / chunk;
+  const int64_t tiles = (chunk + kWriteTileElems - 1) / kWriteTileElems;
+  if (n_chunks * tiles > 0x7fffffffLL) {
+    set_error("rg_scale_cast_single: %lld elements exceed one launch", (long long)numel);
+    return RG_EINVAL;
+  }
+  PassArgs a;
+  memset(&a, 0, sizeof(a));
+  a.single.src = src_dev;
+  a.single.dst = dst_dev;
+  a.single.src_dtype = (int16_t)src_dtype;
+  a.single.dst_dtype = (int16_t)dst_dtype;
+  a.single_numel = numel;
+  a.single_chunk_elems = chunk;
+  a.n_chunks = n_chunks;
+  a.tile_elems = kWriteTileElems;
+  a.tiles_per_chunk = (int32_t)tiles;
+  a.scale = scale;
+  a.zero_fill = src_dev == nullptr ? 1 : 0;
+  DeviceGuard guard(device);
+  const bool streaming = numel * (ss + ds) > ((int64_t)256 << 20);
+  RG_HIP(launch_pass(kModeWrite, a, streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }
 

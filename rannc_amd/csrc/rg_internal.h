@@ -79,7 +79,10 @@ constexpr int64_t kMaxChunkElems = 1 << 20;
 enum : int { kModeReduce = 1, kModeWrite = 2 };
 
 struct PassArgs {
-  const ChunkRec* chunks;        // [n_chunks]
+  const ChunkRec* chunks;        // [n_chunks]; null = one tensor described by `single`
+  ChunkRec single;               // whole-tensor pointers and types (len unused)
+  int64_t single_numel;
+  int64_t single_chunk_elems;
   double* chunk_sumsq;           // [n_chunks] written when reducing
   int32_t* chunk_bad;            // [n_chunks] written when reducing
   const StepResult* result;      // non-null: take coef / overflow gate from the device
@@ -108,6 +111,7 @@ struct FinalizeArgs {
 // streaming: nontemporal loads/stores (data far larger than the caches).
 hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream);
+hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
 
 void set_error(const char* fmt, ...);

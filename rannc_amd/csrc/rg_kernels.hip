@@ -91,15 +91,25 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return ((u & 0x7fffffffu) > 0x7f800000u) ? 0x7fc0u : r;
 }
 
+// fp16 <-> fp32 conversions are kept apart from the neighbouring multiplies: left alone the
+// compiler folds `(_Float16)(x * s)` into a mixed-precision fma with a +0 addend, which
+// turns a -0 product into +0.  The empty asm makes the fp32 value opaque at that point.
+__device__ __forceinline__ float opaque(float f) {
+  asm("" : "+v"(f));
+  return f;
+}
+__device__ __forceinline__ _Float16 f32_to_f16(float f) { return (_Float16)opaque(f); }
+__device__ __forceinline__ float f16_to_f32(_Float16 h) { return opaque((float)h); }
+
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
-  return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f);
+  return (uint32_t)__builtin_bit_cast(unsigned short, f32_to_f16(f));
 }
 
 template <int DT> __device__ __forceinline__ void unpack_word(uint32_t w, float& lo, float& hi);
 template <> __device__ __forceinline__ void unpack_word<RG_F16>(uint32_t w, float& lo, float& hi) {
   const f16x2 h = __builtin_bit_cast(f16x2, w);   // bit_cast needs a scalar, not a vector-element lvalue
-  lo = (float)h.x;
-  hi = (float)h.y;
+  lo = f16_to_f32(h.x);
+  hi = f16_to_f32(h.y);
 }
 template <> __device__ __forceinline__ void unpack_word<RG_BF16>(uint32_t w, float& lo, float& hi) {
   lo = __uint_as_float(w << 16);
@@ -143,7 +153,7 @@ template <> struct Codec<RG_F32, 4> {
 
 // The value as it reads back from a destination of type DT.
 template <int DT> __device__ __forceinline__ float round_dst(float v) { return v; }
-template <> __device__ __forceinline__ float round_dst<RG_F16>(float v) { return (float)(_Float16)v; }
+template <> __device__ __forceinline__ float round_dst<RG_F16>(float v) { return f16_to_f32(f32_to_f16(v)); }
 template <> __device__ __forceinline__ float round_dst<RG_BF16>(float v) {
   return bf16_bits_to_f32(f32_to_bf16_bits(v));
 }
@@ -152,7 +162,7 @@ template <int DT> __device__ __forceinline__ float load1(const char* p) {
   return *reinterpret_cast<const float*>(p);
 }
 template <> __device__ __forceinline__ float load1<RG_F16>(const char* p) {
-  return (float)*reinterpret_cast<const _Float16*>(p);
+  return f16_to_f32(*reinterpret_cast<const _Float16*>(p));
 }
 template <> __device__ __forceinline__ float load1<RG_BF16>(const char* p) {
   return bf16_bits_to_f32(*reinterpret_cast<const unsigned short*>(p));
@@ -161,7 +171,7 @@ template <int DT> __device__ __forceinline__ void store1(char* p, float v) {
   *reinterpret_cast<float*>(p) = v;
 }
 template <> __device__ __forceinline__ void store1<RG_F16>(char* p, float v) {
-  *reinterpret_cast<_Float16*>(p) = (_Float16)v;
+  *reinterpret_cast<_Float16*>(p) = f32_to_f16(v);
 }
 template <> __device__ __forceinline__ void store1<RG_BF16>(char* p, float v) {
   *reinterpret_cast<unsigned short*>(p) = (unsigned short)f32_to_bf16_bits(v);
@@ -309,7 +319,18 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
     coef = a.result->coef;
   }
 
-  const ChunkRec rec = a.chunks[c];
+  ChunkRec rec;
+  if (a.chunks != nullptr) {
+    rec = a.chunks[c];
+  } else {
+    // plan-free launch over one tensor: chunk c is a fixed-size slice of it
+    rec = a.single;
+    const int64_t first = c * a.single_chunk_elems;
+    const int64_t rest = a.single_numel - first;
+    rec.len = (int32_t)(rest < a.single_chunk_elems ? rest : a.single_chunk_elems);
+    if (rec.src) rec.src = reinterpret_cast<const char*>(rec.src) + first * (rec.src_dtype == RG_F32 ? 4 : 2);
+    rec.dst = reinterpret_cast<char*>(rec.dst) + first * (rec.dst_dtype == RG_F32 ? 4 : 2);
+  }
   const int start = tile * a.tile_elems;
   if (start >= rec.len && tile > 0) return;
   const int len = rec.len - start < a.tile_elems ? rec.len - start : a.tile_elems;
@@ -489,6 +510,11 @@ hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t 
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream) {
   if (a.n_tensors > 0)
     hipLaunchKernelGGL(finalize_tensors_kernel, dim3((unsigned)a.n_tensors), dim3(kBlockThreads), 0, stream, a);
+  hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
   return hipGetLastError();
 }

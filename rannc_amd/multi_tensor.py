@@ -122,6 +122,12 @@ class TensorPlan:
     def fused_step(self, inv_scale: float, max_norm: float, flags: int = _lib.RG_STEP_DEFAULT) -> None:
         self.plan.fused_step(inv_scale, max_norm, flags, self._stream())
 
+    def step_begin(self, inv_scale: float) -> None:
+        self.plan.step_begin(inv_scale, self._stream())
+
+    def step_finish(self, max_norm: float, flags: int = _lib.RG_STEP_DEFAULT) -> None:
+        self.plan.step_finish(max_norm, flags, self._stream())
+
     def unscale_pack(self, inv_scale: float) -> None:
         self.plan.unscale_pack(inv_scale, self._stream())
 
@@ -151,3 +157,20 @@ def fill_zero_(t: torch.Tensor) -> torch.Tensor:
     if t.numel():
         _lib.fill_zero(int(t.data_ptr()), t.numel() * t.element_size(), t.device.index, stream_handle(t.device))
     return t
+
+
+def copy_cast_(dst: torch.Tensor, src: Optional[torch.Tensor], scale: float = 1.0) -> torch.Tensor:
+    """``dst.copy_(src)`` (with dtype conversion, optionally scaled) for one pair of contiguous
+    GPU tensors, without building a table; ``src is None`` stores zeros."""
+    if not dst.is_cuda or not dst.is_contiguous():
+        raise ValueError("copy_cast_ needs a contiguous GPU destination")
+    if src is not None:
+        if src.device != dst.device or not src.is_contiguous():
+            raise ValueError("copy_cast_ needs a contiguous source on the destination's device")
+        if src.numel() != dst.numel():
+            raise ValueError(f"copy_cast_: source has {src.numel()} elements, destination {dst.numel()}")
+    if dst.numel():
+        sdt = dtype_code(src.dtype if src is not None else dst.dtype)
+        _lib.scale_cast_single(int(src.data_ptr()) if src is not None else None, int(dst.data_ptr()), dst.numel(),
+                               sdt, dtype_code(dst.dtype), scale, dst.device.index, stream_handle(dst.device))
+    return dst

@@ -1,0 +1,222 @@
+"""GPU parity of the remaining multi-tensor operations against the CPU oracle:
+scale/cast copies for every dtype pair, zero fill, read-only norm, one-pass unscale+pack,
+the plan-free single-tensor entry point, pointer updates and the two-call step."""
+import math
+
+import pytest
+import torch
+
+from oracle import gradpath as oracle
+from rannc_amd import _lib
+from rannc_amd.multi_tensor import TensorPlan, copy_cast_, fill_zero_
+from tests.helpers import TORCH_DTYPE, assert_bits_equal, place_in_arena
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PAIRS = [(s, d) for s in ("f32", "f16", "bf16") for d in ("f32", "f16", "bf16")]
+SHAPES = [(0,), (1,), (5,), (8,), (63,), (64,), (65,), (127,), (1023,), (1024,), (1025,), (2047,), (3, 1000), (16385,), (70001,)]
+
+
+def special_values(dtype):
+    vals = [0.0, -0.0, 1.0, -1.0, 65504.0, 65520.0, 70000.0, 1e-8, 5.96e-8, 2.98e-8, 6.1e-5, 3.4e38, -3.4e38,
+            1e-40, float("inf"), float("-inf"), float("nan"), 1.0 + 2 ** -8, 1.0 + 2 ** -9, 1.0 + 3 * 2 ** -9,
+            1.0 + 2 ** -11, 1.0 + 3 * 2 ** -11, 0.1, 1 / 3]
+    return torch.tensor(vals, dtype=torch.float32).to(dtype)
+
+
+def _inputs(dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    ts = [(torch.randn(s, generator=g) * 10 ** float(torch.randint(-6, 6, (1,), generator=g))).to(dtype) for s in SHAPES]
+    ts.append(special_values(dtype))
+    return ts
+
+
+@pytest.mark.parametrize("src_name,dst_name", PAIRS)
+@pytest.mark.parametrize("scale", [1.0, 0.37])
+def test_scale_cast_all_pairs(src_name, dst_name, scale):
+    sdt, ddt = TORCH_DTYPE[src_name], TORCH_DTYPE[dst_name]
+    srcs_cpu = _inputs(sdt, 11)
+    srcs = place_in_arena(srcs_cpu, DEV, 1, 3)
+    dsts = place_in_arena([torch.full(t.shape, 9.0, dtype=ddt) for t in srcs_cpu], DEV, 3, 1, fill=9.0)
+    plan = TensorPlan(srcs, dsts, chunk_elems=2048)
+    plan.scale_cast(scale)
+    torch.cuda.synchronize()
+    for s, d in zip(srcs_cpu, dsts):
+        if scale == 1.0:
+            want = oracle.cast(s, ddt)
+        else:
+            want = (s.float() * torch.tensor(scale)).to(ddt)
+        assert_bits_equal(d.cpu(), want, f"{src_name}->{dst_name}")
+    plan.close()
+
+
+def test_same_dtype_copy_preserves_every_bit_pattern():
+    # raw copy: NaN payloads and signalling NaNs included
+    bits = torch.arange(-2 ** 15, 2 ** 15, dtype=torch.int32).to(torch.int16)
+    for dt in (torch.float16, torch.bfloat16):
+        src = bits.view(dt).to(DEV)
+        dst = torch.zeros_like(src)
+        TensorPlan([src], [dst]).scale_cast(1.0)
+        assert torch.equal(dst.cpu().view(torch.int16), bits)
+    f = torch.tensor([0x7F800001, 0x7FC00000, 0xFFC12345, 0x00000001, 0x80000000], dtype=torch.int64).to(torch.int32)
+    src = f.view(torch.float32).to(DEV)
+    dst = torch.zeros_like(src)
+    TensorPlan([src], [dst]).scale_cast(1.0)
+    assert torch.equal(dst.cpu().view(torch.int32), f)
+
+
+@pytest.mark.parametrize("dst_name", ["f32", "f16", "bf16"])
+def test_zero_fills_only_the_destinations(dst_name):
+    ddt = TORCH_DTYPE[dst_name]
+    shapes = [(0,), (1,), (7,), (100,), (5000,), (70001,)]
+    dsts = place_in_arena([torch.full(s, 3.0, dtype=ddt) for s in shapes], DEV, 5, 2, fill=3.0)
+    arena_before = dsts[0].untyped_storage()
+    plan = TensorPlan([None] * len(dsts), dsts, chunk_elems=2048)
+    plan.zero()
+    torch.cuda.synchronize()
+    for d in dsts:
+        assert bool((d == 0).all())
+    whole = torch.empty(0, dtype=ddt, device=DEV).set_(arena_before)
+    total = sum(d.numel() for d in dsts)
+    assert int((whole == 3.0).sum()) == whole.numel() - total     # gaps untouched
+    t = torch.full((12345,), 2.0, device=DEV)[1:]
+    fill_zero_(t.contiguous())
+
+
+@pytest.mark.parametrize("src_name", ["f32", "f16", "bf16"])
+def test_grad_norm_measures_the_source_as_stored(src_name):
+    sdt = TORCH_DTYPE[src_name]
+    g = torch.Generator().manual_seed(12)
+    cpu = [(torch.randn(s, generator=g)).to(sdt) for s in SHAPES]
+    dev = place_in_arena(cpu, DEV, 1, 1)
+    # destination dtype differs on purpose: it must not influence the norm of the source
+    dsts = [torch.empty(t.shape, dtype=torch.bfloat16 if sdt != torch.bfloat16 else torch.float16, device=DEV) for t in cpu]
+    plan = TensorPlan(dev, dsts, chunk_elems=4096)
+    plan.grad_norm()
+    res = plan.result()
+    want = oracle.per_tensor_norms(cpu)
+    for a, b in zip(plan.tensor_norms(), want):
+        assert math.isclose(a, b, rel_tol=1e-6, abs_tol=1e-30)
+    assert math.isclose(res.norm, oracle.grad_global_l2_norm(cpu), rel_tol=1e-6)
+    assert res.overflow == 0 and res.clipped == 0
+    plan.close()
+    # norm-only plan without destinations
+    plan = TensorPlan(dev)
+    plan.grad_norm()
+    assert math.isclose(plan.result().norm, oracle.grad_global_l2_norm(cpu), rel_tol=1e-6)
+
+
+def test_norm_closed_forms_on_device():
+    a = torch.full((4096,), 0.5, device=DEV)
+    b = torch.full((64, 64), -0.25, dtype=torch.bfloat16, device=DEV)
+    plan = TensorPlan([a, b])
+    plan.grad_norm()
+    assert plan.tensor_norms() == [32.0, 16.0]
+    assert plan.result().norm == math.sqrt(32.0 ** 2 + 16.0 ** 2)
+
+
+@pytest.mark.parametrize("src_name,dst_name", [("f16", "f32"), ("bf16", "f32"), ("f32", "f32"), ("f16", "f16")])
+def test_unscale_pack_matches_apex_semantics(src_name, dst_name):
+    sdt, ddt = TORCH_DTYPE[src_name], TORCH_DTYPE[dst_name]
+    g = torch.Generator().manual_seed(13)
+    cpu = [(torch.randn(s, generator=g) * 128.0).to(sdt) for s in SHAPES]
+    dev = place_in_arena(cpu, DEV, 1, 1)
+    dsts = place_in_arena([torch.zeros(t.shape, dtype=ddt) for t in cpu], DEV, 2, 1)
+    plan = TensorPlan(dev, dsts, chunk_elems=2048)
+    plan.unscale_pack(1.0 / 128.0)
+    res = plan.result()
+    want, flag = oracle.unscale_and_check(cpu, 1.0 / 128.0, ddt)
+    assert res.overflow == flag == 0
+    for d, w in zip(dsts, want):
+        assert_bits_equal(d.cpu(), w, "unscale_pack")
+    assert math.isclose(res.norm, oracle.grad_global_l2_norm(want), rel_tol=1e-6)
+    # with a non-finite input the values are still written (Apex writes them) and the flag is set
+    cpu[3][2] = float("inf")
+    dev[3].copy_(cpu[3])
+    plan.unscale_pack(1.0 / 128.0)
+    res = plan.result()
+    want, flag = oracle.unscale_and_check(cpu, 1.0 / 128.0, ddt)
+    assert res.overflow == flag == 1
+    for d, w in zip(dsts, want):
+        assert_bits_equal(d.cpu(), w, "unscale_pack overflow")
+    plan.close()
+
+
+@pytest.mark.parametrize("src_name,dst_name", PAIRS)
+def test_single_tensor_entry_point(src_name, dst_name):
+    sdt, ddt = TORCH_DTYPE[src_name], TORCH_DTYPE[dst_name]
+    g = torch.Generator().manual_seed(14)
+    for n in (0, 1, 1023, 1024, 16384, 16385, 100003):
+        s = (torch.randn(n + 1, generator=g) * 3).to(sdt)
+        sd = s.to(DEV)[1:]                       # off the allocation's alignment
+        dd = torch.full((n + 2,), 5.0, dtype=ddt, device=DEV)
+        copy_cast_(dd[1:n + 1], sd)
+        out = dd.cpu()
+        assert_bits_equal(out[1:n + 1], oracle.cast(s[1:], ddt), "single")
+        assert out[0] == 5.0 and out[n + 1] == 5.0
+    z = torch.full((5001,), 5.0, dtype=ddt, device=DEV)
+    copy_cast_(z[1:], None)
+    assert float(z[0]) == 5.0 and bool((z[1:] == 0).all())
+
+
+def test_pointer_update_moves_the_table():
+    g = torch.Generator().manual_seed(15)
+    a = [torch.randn(3000, generator=g), torch.randn(17, generator=g)]
+    b = [torch.randn(3000, generator=g), torch.randn(17, generator=g)]
+    da, db = [t.to(DEV) for t in a], [t.to(DEV) for t in b]
+    out1 = [torch.zeros_like(t) for t in da]
+    out2 = [torch.zeros_like(t) for t in da]
+    plan = TensorPlan(da, out1)
+    plan.scale_cast(2.0)
+    plan.update(srcs=db, dsts=out2)
+    plan.scale_cast(2.0)
+    plan.update(srcs=da)
+    plan.scale_cast(0.5)
+    torch.cuda.synchronize()
+    for x, o in zip(a, out1):
+        assert_bits_equal(o.cpu(), x * 2.0, "first table")
+    for x, o in zip(a, out2):
+        assert_bits_equal(o.cpu(), x * 0.5, "third call overwrote the second")
+    with pytest.raises(ValueError):
+        plan.update(srcs=[da[0][:10], da[1]])
+
+
+def test_two_call_step_equals_fused_step():
+    g = torch.Generator().manual_seed(16)
+    cpu = [(torch.randn(s, generator=g) * 1e-2 * 1024).to(torch.float16) for s in [(50000,), (33,), (4096,)]]
+    dev = [t.to(DEV) for t in cpu]
+    o1 = [torch.zeros(t.shape, device=DEV) for t in cpu]
+    o2 = [torch.zeros(t.shape, device=DEV) for t in cpu]
+    p1, p2 = TensorPlan(dev, o1), TensorPlan(dev, o2)
+    p1.fused_step(1 / 1024.0, 0.3)
+    p2.step_begin(1 / 1024.0)
+    mid = p2.result()
+    assert mid.clipped == 0 and mid.coef == 1.0 and mid.overflow == 0
+    p2.step_finish(0.3)
+    r1, r2 = p1.result(), p2.result()
+    assert (r1.norm, r1.coef, r1.clipped) == (r2.norm, r2.coef, r2.clipped) and r1.clipped == 1
+    for a, b in zip(o1, o2):
+        assert_bits_equal(a.cpu(), b.cpu(), "two-call")
+    with pytest.raises(ValueError, match="pending"):
+        p2.step_finish(0.3)
+
+
+def test_error_paths():
+    a = torch.zeros(10, device=DEV)
+    with pytest.raises(ValueError, match="contiguous"):
+        TensorPlan([torch.zeros(10, 10, device=DEV).t()], [torch.zeros(10, 10, device=DEV)])
+    with pytest.raises(ValueError, match="GPU"):
+        TensorPlan([torch.zeros(10)], [a])
+    with pytest.raises(ValueError, match="elements"):
+        TensorPlan([a], [torch.zeros(11, device=DEV)])
+    with pytest.raises(ValueError, match="dtype"):
+        TensorPlan([torch.zeros(10, dtype=torch.float64, device=DEV)], [a])
+    p = TensorPlan([a])
+    with pytest.raises(ValueError, match="destination"):
+        p.scale_cast(1.0)
+    with pytest.raises(ValueError, match="inv_scale"):
+        TensorPlan([a], [torch.zeros(10, device=DEV)]).fused_step(0.0, 1.0)
+    with pytest.raises(ValueError, match="in place"):
+        TensorPlan([a], [a.view(torch.int32).view(torch.float32)]).plan  # same dtype in place is fine
+        b16 = torch.zeros(20, dtype=torch.bfloat16, device=DEV)
+        _lib.scale_cast_single(b16.data_ptr(), b16.data_ptr(), 10, _lib.RG_BF16, _lib.RG_F32, 1.0, 0, 0)
