@@ -48,6 +48,7 @@ class _AmpStash:
         self.all_fp32_from_fp16_params: List[torch.Tensor] = []
         self.all_fp32_from_fp32_params: List[torch.Tensor] = []
         self.already_patched = False
+        self.lazy_init_called = False
         self.unscale_plan: Optional[TensorPlan] = None
         self.unscale_key: Optional[tuple] = None
         self.copy_back_plan: Optional[TensorPlan] = None
@@ -148,6 +149,22 @@ def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_lev
                 mod._buffers[name] = b.to(half_dtype)
     stash = _AmpStash()
     stash.fused = fused
+    optimizer._amp_stash = stash
+    scaler = LossScaler(loss_scale, min_loss_scale=min_loss_scale, max_loss_scale=max_loss_scale)
+    _amp_state.loss_scalers = [scaler]
+    _amp_state.opt_level = opt_level
+    _patch_step(optimizer)
+    return model, optimizer
+
+
+def _lazy_init_maybe_master_weights(optimizer: torch.optim.Optimizer) -> None:
+    """Create the fp32 masters and re-point the optimizer at them.  As in Apex this happens
+    lazily, at the first ``scale_loss``: by then ``patch_optimizer`` has replaced the
+    optimizer's parameters by the ones this process owns (ZeRO: their local segments)."""
+    stash = optimizer._amp_stash
+    if stash.lazy_init_called:
+        return
+    stash.lazy_init_called = True
     for group in optimizer.param_groups:
         new_params = []
         for p in group["params"]:
@@ -163,12 +180,6 @@ def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_lev
                 stash.all_fp32_from_fp32_params.append(p)
                 new_params.append(p)
         group["params"] = new_params
-    optimizer._amp_stash = stash
-    scaler = LossScaler(loss_scale, min_loss_scale=min_loss_scale, max_loss_scale=max_loss_scale)
-    _amp_state.loss_scalers = [scaler]
-    _amp_state.opt_level = opt_level
-    _patch_step(optimizer)
-    return model, optimizer
 
 
 def master_params(optimizer: torch.optim.Optimizer) -> Iterator[torch.Tensor]:
@@ -229,6 +240,7 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
     loss scale, and arm a one-shot skip of ``optimizer.step`` after an overflow."""
     scaler = _amp_state.loss_scalers[0]
     stash = optimizer._amp_stash
+    _lazy_init_maybe_master_weights(optimizer)
     yield loss.float() * scaler.loss_scale()
     model_grads, master_grads = [], []
     if stash.master_grad_bucket is None and stash.all_fp32_from_fp16_params:
@@ -266,6 +278,7 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
 # --------------------------------------------------------------------------- reference API
 
 def zip_params(optimizer):
+    _lazy_init_maybe_master_weights(optimizer)
     stash = optimizer._amp_stash
     return zip(stash.all_fp32_from_fp16_params, stash.all_fp16_params)
 

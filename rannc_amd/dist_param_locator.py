@@ -38,10 +38,18 @@ class DistributedParamLocator:
         self.shapes[pid] = param.shape
         self.requires_grad[pid] = bool(param.requires_grad)
         off, src = lay[2][self.rank], lay[3][self.rank]
-        part = torch.empty(src, dtype=param.dtype, device=param.device)
-        if src > 0:
-            with torch.no_grad():
-                copy_cast_(part, param.detach().contiguous().view(-1).narrow(0, off, src))
+        flat = param.detach().contiguous().view(-1).narrow(0, off, src)
+        if param.is_cuda:
+            part = torch.empty(src, dtype=param.dtype, device=param.device)
+            if src > 0:
+                with torch.no_grad():
+                    copy_cast_(part, flat)
+        else:
+            # A parameter still on the host (modules are built there): its slice is uploaded,
+            # which is a transfer and not arithmetic, and the segment lives on the GPU.
+            if not torch.cuda.is_available():
+                raise RuntimeError("store_dist_param needs a GPU: segments are kept in device memory")
+            part = flat.to(torch.device("cuda", torch.cuda.current_device()))
         part.requires_grad_(param.requires_grad)
         self.param_parts[pid] = part
         return part
