@@ -267,8 +267,11 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   const size_t nt = (size_t)(n > 0 ? n : 1), nc = (size_t)(p->n_chunks > 0 ? p->n_chunks : 1);
   const size_t o_chunks = carve(nc * sizeof(ChunkRec));
   const size_t o_begin = carve((nt + 1) * sizeof(int64_t));
-  const size_t o_sumsq = carve(nc * sizeof(double));
-  const size_t o_bad = carve(nc * sizeof(int32_t));
+  // a tiled reduce+write pass leaves one partial per tile
+  if (p->write_tile_elems < kMinWriteTileElems) p->write_tile_elems = kMinWriteTileElems;
+  const size_t max_tiles = (size_t)((p->chunk_elems + p->write_tile_elems - 1) / p->write_tile_elems);
+  const size_t o_sumsq = carve(nc * max_tiles * sizeof(double));
+  const size_t o_bad = carve(nc * max_tiles * sizeof(int32_t));
   const size_t o_tnorm = carve(nt * sizeof(float));
   const size_t o_tsq = carve(nt * sizeof(double));
   const size_t o_tbad = carve(nt * sizeof(int32_t));
@@ -399,8 +402,9 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   return a;
 }
 
-static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_overflow) {
+static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_overflow, int partials_per_chunk = 1) {
   FinalizeArgs f;
+  f.partials_per_chunk = partials_per_chunk;
   f.tensor_chunk_begin = p->d_tensor_chunk_begin;
   f.chunk_sumsq = p->d_chunk_sumsq;
   f.chunk_bad = p->d_chunk_bad;
@@ -416,7 +420,8 @@ static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_o
 
 // Write-only passes cut every chunk into tiles so that more, smaller blocks are in flight.
 static void split_for_write(const rg_plan* p, PassArgs& a) {
-  const int64_t tile = p->write_tile_elems;
+  int64_t tile = p->write_tile_elems;
+  if (tile > 0 && tile < kMinWriteTileElems) tile = kMinWriteTileElems;
   if (tile > 0 && tile < p->chunk_elems && p->n_chunks * ((p->chunk_elems + tile - 1) / tile) <= 0x7fffffffLL) {
     a.tile_elems = (int32_t)tile;
     a.tiles_per_chunk = (int32_t)((p->chunk_elems + tile - 1) / tile);
@@ -514,8 +519,10 @@ RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   }
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  RG_HIP(launch_pass(kModeReduce | kModeWrite, pass_args(p, inv_scale), p->streaming, s));
-  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
+  PassArgs a = pass_args(p, inv_scale);
+  split_for_write(p, a);
+  RG_HIP(launch_pass(kModeReduce | kModeWrite, a, p->streaming, s));
+  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0, a.tiles_per_chunk), s));
   return RG_OK;
 }
 

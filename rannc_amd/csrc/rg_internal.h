@@ -60,6 +60,9 @@ static_assert(sizeof(StepResult) == 32, "result block must stay 32 bytes");
 #ifndef RG_ALIGN_BYTES
 #define RG_ALIGN_BYTES 128
 #endif
+#ifndef RG_WRITE_ALIGN_BYTES
+#define RG_WRITE_ALIGN_BYTES 2
+#endif
 #ifndef RG_DEFAULT_CHUNK_ELEMS
 #define RG_DEFAULT_CHUNK_ELEMS 16384
 #endif
@@ -71,9 +74,16 @@ constexpr int kReduceElemsPerThread = RG_REDUCE_ELEMS_PER_THREAD;
 constexpr int kWriteElemsPerThread = RG_WRITE_ELEMS_PER_THREAD;
 constexpr int kWriteThreads = RG_WRITE_THREADS;                  // block size of write-only passes
 constexpr int kWriteTileElems = RG_WRITE_TILE_ELEMS;             // writing passes cut each chunk into tiles of this size
-constexpr unsigned kAlignBytes = RG_ALIGN_BYTES;                 // per-chunk peel of the written (or read-only) side
+// Per-chunk peel.  The read-only pass peels its source to 128 bytes (one scalar head per
+// 16K-element chunk).  Passes that write do not peel at all (2 = element alignment): gfx950
+// executes element-aligned 128-bit stores, and measured on MI355X that beats peeling the
+// destination to a line boundary (6.1-6.2 vs 5.3-5.7 TB/s for an odd-offset destination),
+// because the scalar head is a dependent load->store round trip inside a very short tile.
+constexpr unsigned kAlignBytes = RG_ALIGN_BYTES;
+constexpr unsigned kWriteAlignBytes = RG_WRITE_ALIGN_BYTES;
 constexpr int64_t kChunkQuantum = 2048;    // chunk sizes are multiples of this many elements
 constexpr int64_t kMaxChunkElems = 1 << 20;
+constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan
 
 // Pass selection for the chunk kernel.
 enum : int { kModeReduce = 1, kModeWrite = 2 };
@@ -83,8 +93,8 @@ struct PassArgs {
   ChunkRec single;               // whole-tensor pointers and types (len unused)
   int64_t single_numel;
   int64_t single_chunk_elems;
-  double* chunk_sumsq;           // [n_chunks] written when reducing
-  int32_t* chunk_bad;            // [n_chunks] written when reducing
+  double* chunk_sumsq;           // [n_chunks * tiles_per_chunk] written when reducing
+  int32_t* chunk_bad;            // [n_chunks * tiles_per_chunk] written when reducing
   const StepResult* result;      // non-null: take coef / overflow gate from the device
   int64_t n_chunks;
   int32_t tile_elems;            // elements one block handles (== chunk_elems unless the pass splits chunks)
@@ -104,6 +114,7 @@ struct FinalizeArgs {
   int32_t* tensor_bad;                // [n_tensors]
   StepResult* result;
   int32_t n_tensors;
+  int32_t partials_per_chunk;         // 1, or the tile count when the reducing pass was tiled
   float max_norm;
   int32_t ignore_overflow;  // overflow is reported but neither gates the clip nor the write
 };

@@ -8,10 +8,9 @@
 // Inside a chunk every load and store instruction is contiguous across the wavefront: a
 // lane moves E consecutive elements per instruction, E = 4 when either side is fp32 and 8
 // otherwise, so the wider side always moves 16 bytes per lane (1 KiB per wavefront
-// instruction) and the narrower side 8.  The side that is written (for a read-only pass,
-// the side that is read) is peeled to a 128-byte boundary per chunk, so streaming stores
-// cover whole lines; the other side is accessed at its natural element alignment, which
-// gfx950 serves with the same instructions.
+// instruction) and the narrower side 8.  Accesses only need element alignment: gfx950
+// executes 2-byte-aligned 64/128-bit loads and stores.  The read-only pass still peels its
+// source to a 128-byte boundary per chunk; passes that write do not peel (see rg_internal.h).
 //
 // Plans whose data is far larger than the caches use nontemporal loads and stores: measured
 // on MI355X that lifts a read-only pass from 6.3 to 7.1 TB/s, and nontemporal stores keep
@@ -34,8 +33,8 @@ typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
 
-// Block size of a pass: write-only passes may use smaller blocks than reducing ones.
-template <int MODE> struct PassThreads { static constexpr int value = (MODE == kModeWrite) ? kWriteThreads : kBlockThreads; };
+// Block size of a pass: passes that write use smaller blocks than the read-only one.
+template <int MODE> struct PassThreads { static constexpr int value = (MODE & kModeWrite) ? kWriteThreads : kBlockThreads; };
 
 template <int DT> struct ElemSize { static constexpr int value = 2; };
 template <> struct ElemSize<RG_F32> { static constexpr int value = 4; };
@@ -58,14 +57,15 @@ template <bool NT> __device__ __forceinline__ u32x4 ld16_a2(const char* p) {
 template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
   return NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x2_a2*>(p)) : *reinterpret_cast<const u32x2_a2*>(p);
 }
-// Stores are aligned to their own size (the chunk head is peeled for that).
+// Stores: the pointer type promises element alignment only (what the peel guarantees beyond
+// that is a performance matter, not a correctness one).
 template <bool NT> __device__ __forceinline__ void st16(char* p, u32x4 v) {
-  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
-  else *reinterpret_cast<u32x4*>(p) = v;
+  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_a2*>(p));
+  else *reinterpret_cast<u32x4_a2*>(p) = v;
 }
 template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
-  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
-  else *reinterpret_cast<u32x2*>(p) = v;
+  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x2_a2*>(p));
+  else *reinterpret_cast<u32x2_a2*>(p) = v;
 }
 
 template <int DT, int E, bool NT> struct Mem;
@@ -203,26 +203,41 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   constexpr int kPerThread = kWrite ? kWriteElemsPerThread : kReduceElemsPerThread;
   constexpr int U = kPerThread >= E ? kPerThread / E : 1;      // instructions in flight per lane
   constexpr int AS = kWrite ? DS : SS;
+  constexpr unsigned kPeel = kWrite ? kWriteAlignBytes : kAlignBytes;
   const uintptr_t a = kWrite ? reinterpret_cast<uintptr_t>(dp) : reinterpret_cast<uintptr_t>(sp);
-  int head = (int)(((kAlignBytes - (unsigned)(a & (kAlignBytes - 1))) & (kAlignBytes - 1)) / (unsigned)AS);
+  int head = (int)(((kPeel - (unsigned)(a & (kPeel - 1))) & (kPeel - 1)) / (unsigned)AS);
   if (head > len) head = len;
   const int nbody = (len - head) / E * E;
   const int tail0 = head + nbody;
   const int tid = threadIdx.x;
 
-  // Unaligned head (< 128 bytes) and ragged tail (< E elements): one element per thread.
+  // Unaligned head (read-only pass: < 128 bytes) and ragged tail (< E elements): one element per thread.
+  // The element is loaded here, before the vector loop, and converted and stored after it,
+  // so its memory latency overlaps the vector loads instead of preceding them.
   const int nscalar = head + (len - tail0);
-  for (int k = tid; k < nscalar; k += T) {
-    const int i = k < head ? k : tail0 + (k - head);
+  auto scalar_index = [&](int k) { return k < head ? k : tail0 + (k - head); };
+  auto scalar_load = [&](int i) -> uint32_t {
+    return SS == 4 ? *reinterpret_cast<const uint32_t*>(sp + (size_t)i * 4)
+                   : (uint32_t)*reinterpret_cast<const unsigned short*>(sp + (size_t)i * 2);
+  };
+  auto scalar_finish = [&](uint32_t raw, int i) {
     if (S == D && raw_copy) {
-      if (SS == 4) *reinterpret_cast<uint32_t*>(dp + (size_t)i * 4) = *reinterpret_cast<const uint32_t*>(sp + (size_t)i * 4);
-      else *reinterpret_cast<unsigned short*>(dp + (size_t)i * 2) = *reinterpret_cast<const unsigned short*>(sp + (size_t)i * 2);
+      if (SS == 4) *reinterpret_cast<uint32_t*>(dp + (size_t)i * 4) = raw;
+      else *reinterpret_cast<unsigned short*>(dp + (size_t)i * 2) = (unsigned short)raw;
     } else {
-      const float v = round_dst<D>(load1<S>(sp + (size_t)i * SS) * scale);
+      float x;
+      if (S == RG_F32) x = __uint_as_float(raw);
+      else if (S == RG_F16) x = f16_to_f32(__builtin_bit_cast(_Float16, (unsigned short)raw));
+      else x = bf16_bits_to_f32(raw);
+      const float v = round_dst<D>(x * scale);
       if (kReduce) acc[0] = __builtin_fmaf(v, v, acc[0]);
       if (kWrite) store1<D>(dp + (size_t)i * DS, v * coef);
     }
-  }
+  };
+  const bool has_scalar = tid < nscalar;
+  const int scalar_i = has_scalar ? scalar_index(tid) : 0;
+  uint32_t scalar_raw = 0;
+  if (has_scalar) scalar_raw = scalar_load(scalar_i);
 
   const char* sb = sp + (size_t)head * SS;
   char* db = dp + (size_t)head * DS;
@@ -279,13 +294,19 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
       consume(in[u], e, e < nbody);
     }
   }
+
+  if (has_scalar) scalar_finish(scalar_raw, scalar_i);
+  for (int k = tid + T; k < nscalar; k += T) {
+    const int i = scalar_index(k);
+    scalar_finish(scalar_load(i), i);
+  }
 }
 
 // Zero `nbytes` bytes at p (p and nbytes are multiples of 2).
 template <bool NT, int T>
 __device__ __forceinline__ void zero_range(char* p, int nbytes) {
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
-  int head = (int)((kAlignBytes - (unsigned)(a & (kAlignBytes - 1))) & (kAlignBytes - 1));
+  int head = (int)((kWriteAlignBytes - (unsigned)(a & (kWriteAlignBytes - 1))) & (kWriteAlignBytes - 1));
   if (head > nbytes) head = nbytes;
   const int nvec = (nbytes - head) / 16;
   const int tail0 = head + nvec * 16;
@@ -299,19 +320,20 @@ __device__ __forceinline__ void zero_range(char* p, int nbytes) {
   for (int v = tid; v < nvec; v += T) st16<NT>(p + head + (size_t)v * 16, z);
 }
 
-template <int S>
+template <int S, int T>
 __device__ __forceinline__ int rescan_nonfinite(const char* sp, int len) {
   int bad = 0;
-  for (int i = threadIdx.x; i < len; i += kBlockThreads)
+  for (int i = threadIdx.x; i < len; i += T)
     bad |= nonfinite_at<S>(sp + (size_t)i * ElemSize<S>::value) ? 1 : 0;
   return bad;
 }
 
 template <int MODE, bool NT>
 __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs a) {
-  // Block -> (chunk, tile of the chunk).  Reducing passes never split (one partial per chunk).
-  const int64_t c = (MODE & kModeReduce) ? (int64_t)blockIdx.x : (int64_t)(blockIdx.x / (unsigned)a.tiles_per_chunk);
-  const int tile = (MODE & kModeReduce) ? 0 : (int)(blockIdx.x % (unsigned)a.tiles_per_chunk);
+  // Block -> (chunk, tile of the chunk); its partial sum, if any, goes to slot blockIdx.x.
+  constexpr int T = PassThreads<MODE>::value;
+  const int64_t c = (int64_t)(blockIdx.x / (unsigned)a.tiles_per_chunk);
+  const int tile = (int)(blockIdx.x % (unsigned)a.tiles_per_chunk);
   float coef = 1.0f;
   if (a.result != nullptr) {
     // Values produced by the finalize kernel earlier on the same stream.
@@ -331,9 +353,25 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
     if (rec.src) rec.src = reinterpret_cast<const char*>(rec.src) + first * (rec.src_dtype == RG_F32 ? 4 : 2);
     rec.dst = reinterpret_cast<char*>(rec.dst) + first * (rec.dst_dtype == RG_F32 ? 4 : 2);
   }
-  const int start = tile * a.tile_elems;
-  if (start >= rec.len && tile > 0) return;
-  const int len = rec.len - start < a.tile_elems ? rec.len - start : a.tile_elems;
+  // Tiles are laid out from the first peel boundary of the chunk's written side, so only
+  // tile 0 of a chunk can have an unaligned head; the others start aligned.
+  int chunk_head = 0;
+  if (a.tiles_per_chunk > 1 && kWriteAlignBytes > 4) {
+    const unsigned mis = (unsigned)(reinterpret_cast<uintptr_t>(rec.dst) & (kWriteAlignBytes - 1));
+    chunk_head = (int)(((kWriteAlignBytes - mis) & (kWriteAlignBytes - 1)) / (rec.dst_dtype == RG_F32 ? 4u : 2u));
+    if (chunk_head > rec.len) chunk_head = rec.len;
+  }
+  const int start = tile == 0 ? 0 : chunk_head + tile * a.tile_elems;
+  int end = chunk_head + (tile + 1) * a.tile_elems;
+  if (end > rec.len) end = rec.len;
+  if (start >= end) {
+    if ((MODE & kModeReduce) && threadIdx.x == 0) {
+      a.chunk_sumsq[blockIdx.x] = 0.0;
+      a.chunk_bad[blockIdx.x] = 0;
+    }
+    return;
+  }
+  const int len = end - start;
   const char* sp = rec.src ? reinterpret_cast<const char*>(rec.src) + (size_t)start * (rec.src_dtype == RG_F32 ? 4 : 2) : nullptr;
   char* dp = reinterpret_cast<char*>(rec.dst) + (size_t)start * (rec.dst_dtype == RG_F32 ? 4 : 2);
   const int src_kind = rec.src_dtype;
@@ -342,7 +380,7 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (sp == nullptr || a.zero_fill) {
-    if (MODE & kModeWrite) zero_range<NT, PassThreads<MODE>::value>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
+    if (MODE & kModeWrite) zero_range<NT, T>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
   } else {
     switch (src_kind * 3 + dst_kind) {
       case RG_F32 * 3 + RG_F32: process_chunk<RG_F32, RG_F32, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
@@ -358,16 +396,19 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
   }
 
   if (MODE & kModeReduce) {
-    // Fixed-order combine: 8 lanes of the thread, 64 lanes of the wavefront by shuffle,
-    // 4 wavefronts through LDS.  Everything past the per-thread fp32 sums is double.
+    // Fixed-order combine: 8 lanes of the thread, 64 lanes of the wavefront by shuffle, the
+    // wavefronts through LDS in index order.  Everything past the per-thread fp32 sums is double.
+    constexpr int kWaves = T / 64;
     double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
                (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off);
-    __shared__ double wave_sum[kBlockThreads / 64];
+    __shared__ double wave_sum[kWaves];
     if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = s;
     __syncthreads();
-    const double total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+    double total = wave_sum[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) total += wave_sum[w];
     // A non-finite input makes its square, and so the chunk's sum, non-finite; a finite sum
     // therefore proves every input was finite.  Only chunks whose sum is not finite are
     // looked at again element by element (the sum can also overflow from finite inputs).
@@ -375,15 +416,15 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
     if (!(fabs(total) <= 1.79769313486231570e308)) {
       int mine = 0;
       if (sp != nullptr) {
-        if (src_kind == RG_F32) mine = rescan_nonfinite<RG_F32>(sp, len);
-        else if (src_kind == RG_F16) mine = rescan_nonfinite<RG_F16>(sp, len);
-        else mine = rescan_nonfinite<RG_BF16>(sp, len);
+        if (src_kind == RG_F32) mine = rescan_nonfinite<RG_F32, T>(sp, len);
+        else if (src_kind == RG_F16) mine = rescan_nonfinite<RG_F16, T>(sp, len);
+        else mine = rescan_nonfinite<RG_BF16, T>(sp, len);
       }
       bad = __syncthreads_or(mine);
     }
     if (threadIdx.x == 0) {
-      a.chunk_sumsq[c] = total;
-      a.chunk_bad[c] = bad;
+      a.chunk_sumsq[blockIdx.x] = total;
+      a.chunk_bad[blockIdx.x] = bad;
     }
   }
 }
@@ -414,8 +455,8 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_tensors_kernel(Finaliz
   const int t = blockIdx.x;
   double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
   int bad = 0;
-  const int64_t end = a.tensor_chunk_begin[t + 1];
-  int64_t c = a.tensor_chunk_begin[t] + threadIdx.x;
+  const int64_t end = a.tensor_chunk_begin[t + 1] * a.partials_per_chunk;
+  int64_t c = a.tensor_chunk_begin[t] * a.partials_per_chunk + threadIdx.x;
   for (; c + 3 * kBlockThreads < end; c += 4 * kBlockThreads) {
     const double v0 = a.chunk_sumsq[c], v1 = a.chunk_sumsq[c + kBlockThreads];
     const double v2 = a.chunk_sumsq[c + 2 * kBlockThreads], v3 = a.chunk_sumsq[c + 3 * kBlockThreads];
