@@ -137,7 +137,9 @@ def main() -> int:
     for _ in range(args.warmup):
         plan.fused_step(cfg.inv_scale, cfg.max_norm)
     torch.cuda.synchronize()
-    plan.plan.enable_timing(args.steps)
+    # Timed region: HIP events (recorded by the library on the launch stream) bracket only the
+    # dominant kernel, the write pass - each record costs a few microseconds of stream time.
+    plan.plan.enable_timing(-args.steps)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -145,6 +147,12 @@ def main() -> int:
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     res = plan.result()
+    write_only = [plan.plan.read_timing(i) for i in range(args.steps)]
+    # A second, untimed loop brackets all three stages for the breakdown.
+    plan.plan.enable_timing(args.steps)
+    for _ in range(args.steps):
+        plan.fused_step(cfg.inv_scale, cfg.max_norm)
+    torch.cuda.synchronize()
     per_kernel = [plan.plan.read_timing(i) for i in range(args.steps)]
     plan.plan.enable_timing(0)
 
@@ -154,20 +162,21 @@ def main() -> int:
     value = step_bytes / step_s / 1e9
 
     # dominant kernel: the write pass (re-read s*N, write d*N)
-    write_ms = sum(k[2] for k in per_kernel) / len(per_kernel)
+    write_ms = sum(k[2] for k in write_only) / len(write_only)
     reduce_ms = sum(k[0] for k in per_kernel) / len(per_kernel)
     final_ms = sum(k[1] for k in per_kernel) / len(per_kernel)
     write_bytes = (s + d) * n
     achieved = write_bytes / (write_ms * 1e-3) / 1e9
     roofline = {
-        "bound": "hbm", "kernel": "pass_kernel<write>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "bound": "hbm", "kernel": "pass_kernel<write, streaming>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
         "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.key),
         "algorithmic_bytes_per_launch": write_bytes, "avg_launch_ms": round(write_ms, 4),
         "other_kernels": {
             "pass_kernel<reduce>": {"avg_launch_ms": round(reduce_ms, 4), "algorithmic_bytes_per_launch": s * n,
                                     "achieved": round(s * n / (reduce_ms * 1e-3) / 1e9, 1)},
-            "finalize_kernel": {"avg_launch_ms": round(final_ms, 4)},
+            "finalize_tensors_kernel+finalize_total_kernel": {"avg_launch_ms": round(final_ms, 4)},
+            "note": "from a second, untimed loop of the same steps with all stages bracketed",
         },
     }
 

@@ -186,7 +186,9 @@ int rg_read_tensor_norms(rg_plan* plan, float* out_host, void* stream);
  * rg_fused_step records HIP events on its stream around its three kernels into the next
  * slot of a ring; slots == 0 switches it off.  rg_plan_read_timing waits for that slot and
  * returns milliseconds: ms[0] reduce pass, ms[1] finalize, ms[2] write pass, ms[3] whole step.
- * slot counts fused steps since timing was enabled, modulo `slots`. */
+ * slot counts fused steps since timing was enabled, modulo `slots`.
+ * A negative `slots` brackets only the write pass (two records per step instead of four, for
+ * measurements where the records' own cost matters); ms[0], ms[1], ms[3] then read -1. */
 int rg_plan_enable_timing(rg_plan* plan, int slots);
 int rg_plan_read_timing(rg_plan* plan, int slot, float ms[4]);
 

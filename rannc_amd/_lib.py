@@ -214,6 +214,7 @@ class Plan:
         return list(buf)[: self.n]
 
     def enable_timing(self, slots: int) -> None:
+        """slots > 0: bracket all stages of each fused step; < 0: only the write pass; 0: off."""
         check(lib.rg_plan_enable_timing(self._handle, slots))
 
     def read_timing(self, slot: int) -> List[float]:

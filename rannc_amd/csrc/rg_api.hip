@@ -82,6 +82,8 @@ struct rg_plan {
   int64_t* d_tensor_chunk_begin = nullptr;
   double* d_chunk_sumsq = nullptr;
   int32_t* d_chunk_bad = nullptr;
+  double* d_tile_sumsq = nullptr;   // [n_chunks * max_tiles]: partials of a tiled reduce+write pass
+  int32_t* d_tile_bad = nullptr;
   float* d_tensor_norm = nullptr;
   double* d_tensor_sq = nullptr;
   int32_t* d_tensor_bad = nullptr;
@@ -102,6 +104,7 @@ struct rg_plan {
   std::vector<hipEvent_t> timing_events;
   int timing_slots = 0;
   int64_t timing_count = 0;
+  bool timing_all = true;  // false: only the write pass is bracketed (two records per step)
 };
 
 static int check_pointer(const void* p, int esz, const char* which, int i) {
@@ -270,8 +273,10 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   // a tiled reduce+write pass leaves one partial per tile
   if (p->write_tile_elems < kMinWriteTileElems) p->write_tile_elems = kMinWriteTileElems;
   const size_t max_tiles = (size_t)((p->chunk_elems + p->write_tile_elems - 1) / p->write_tile_elems);
-  const size_t o_sumsq = carve(nc * max_tiles * sizeof(double));
-  const size_t o_bad = carve(nc * max_tiles * sizeof(int32_t));
+  const size_t o_sumsq = carve(nc * sizeof(double));
+  const size_t o_bad = carve(nc * sizeof(int32_t));
+  const size_t o_tile_sumsq = carve(nc * max_tiles * sizeof(double));
+  const size_t o_tile_bad = carve(nc * max_tiles * sizeof(int32_t));
   const size_t o_tnorm = carve(nt * sizeof(float));
   const size_t o_tsq = carve(nt * sizeof(double));
   const size_t o_tbad = carve(nt * sizeof(int32_t));
@@ -290,6 +295,8 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->d_tensor_chunk_begin = reinterpret_cast<int64_t*>(b + o_begin);
   p->d_chunk_sumsq = reinterpret_cast<double*>(b + o_sumsq);
   p->d_chunk_bad = reinterpret_cast<int32_t*>(b + o_bad);
+  p->d_tile_sumsq = reinterpret_cast<double*>(b + o_tile_sumsq);
+  p->d_tile_bad = reinterpret_cast<int32_t*>(b + o_tile_bad);
   p->d_tensor_norm = reinterpret_cast<float*>(b + o_tnorm);
   p->d_tensor_sq = reinterpret_cast<double*>(b + o_tsq);
   p->d_tensor_bad = reinterpret_cast<int32_t*>(b + o_tbad);
@@ -402,9 +409,8 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   return a;
 }
 
-static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_overflow, int partials_per_chunk = 1) {
+static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_overflow) {
   FinalizeArgs f;
-  f.partials_per_chunk = partials_per_chunk;
   f.tensor_chunk_begin = p->d_tensor_chunk_begin;
   f.chunk_sumsq = p->d_chunk_sumsq;
   f.chunk_bad = p->d_chunk_bad;
@@ -463,9 +469,10 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   hipEvent_t* ev = nullptr;
   if (p->timing_slots > 0) ev = &p->timing_events[(size_t)(p->timing_count++ % p->timing_slots) * 4];
   PassArgs a = pass_args(p, inv_scale);
-  if (ev) RG_HIP(hipEventRecord(ev[0], s));
+  const bool all = ev != nullptr && p->timing_all;
+  if (all) RG_HIP(hipEventRecord(ev[0], s));
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
-  if (ev) RG_HIP(hipEventRecord(ev[1], s));
+  if (all) RG_HIP(hipEventRecord(ev[1], s));
   RG_HIP(launch_finalize(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
   if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
@@ -521,8 +528,20 @@ RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, inv_scale);
   split_for_write(p, a);
+  if (a.tiles_per_chunk > 1 && a.tile_elems * 2 <= p->chunk_elems) {
+    // every tile of this pass also pays a block-wide reduction: twice the tile amortises it
+    a.tile_elems *= 2;
+    a.tiles_per_chunk = (int32_t)((p->chunk_elems + a.tile_elems - 1) / a.tile_elems);
+  }
+  if (a.tiles_per_chunk > 1) {
+    a.chunk_sumsq = p->d_tile_sumsq;
+    a.chunk_bad = p->d_tile_bad;
+  }
   RG_HIP(launch_pass(kModeReduce | kModeWrite, a, p->streaming, s));
-  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0, a.tiles_per_chunk), s));
+  if (a.tiles_per_chunk > 1)
+    RG_HIP(launch_fold_tiles(p->d_tile_sumsq, p->d_tile_bad, p->d_chunk_sumsq, p->d_chunk_bad, p->n_chunks,
+                             a.tiles_per_chunk, s));
+  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
   return RG_OK;
 }
 
@@ -662,6 +681,10 @@ RG_API int rg_read_tensor_norms(rg_plan* p, float* out_host, void* stream) {
 // ---------------------------------------------------------------------------- timing
 
 RG_API int rg_plan_enable_timing(rg_plan* p, int slots) {
+  // slots < 0: bracket only the write pass (the dominant kernel) in |slots| slots
+  const bool all = slots >= 0;
+  if (slots < 0) slots = -slots;
+  if (p != nullptr) p->timing_all = all;
   if (p == nullptr || slots < 0 || slots > 65536) {
     set_error("rg_plan_enable_timing: bad arguments");
     return RG_EINVAL;
@@ -689,9 +712,12 @@ RG_API int rg_plan_read_timing(rg_plan* p, int slot, float ms[4]) {
   DeviceGuard guard(p->device);
   hipEvent_t* ev = &p->timing_events[(size_t)slot * 4];
   RG_HIP(hipEventSynchronize(ev[3]));
-  RG_HIP(hipEventElapsedTime(&ms[0], ev[0], ev[1]));
-  RG_HIP(hipEventElapsedTime(&ms[1], ev[1], ev[2]));
+  ms[0] = ms[1] = ms[3] = -1.0f;
+  if (p->timing_all) {
+    RG_HIP(hipEventElapsedTime(&ms[0], ev[0], ev[1]));
+    RG_HIP(hipEventElapsedTime(&ms[1], ev[1], ev[2]));
+    RG_HIP(hipEventElapsedTime(&ms[3], ev[0], ev[3]));
+  }
   RG_HIP(hipEventElapsedTime(&ms[2], ev[2], ev[3]));
-  RG_HIP(hipEventElapsedTime(&ms[3], ev[0], ev[3]));
   return RG_OK;
 }

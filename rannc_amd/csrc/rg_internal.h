@@ -114,7 +114,6 @@ struct FinalizeArgs {
   int32_t* tensor_bad;                // [n_tensors]
   StepResult* result;
   int32_t n_tensors;
-  int32_t partials_per_chunk;         // 1, or the tile count when the reducing pass was tiled
   float max_norm;
   int32_t ignore_overflow;  // overflow is reported but neither gates the clip nor the write
 };
@@ -123,6 +122,9 @@ struct FinalizeArgs {
 hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream);
 hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream);
+// chunk[c] = sum over t of tile[c * tiles_per_chunk + t], in order (after a tiled reducing pass)
+hipError_t launch_fold_tiles(const double* tile_sumsq, const int32_t* tile_bad, double* chunk_sumsq, int32_t* chunk_bad,
+                             int64_t n_chunks, int tiles_per_chunk, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
 
 void set_error(const char* fmt, ...);

@@ -84,12 +84,8 @@ template <int DT, bool NT> struct Mem<DT, 8, NT> {   // 16-bit types, 8 elements
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-// Round-to-nearest-even narrowing; NaN becomes the canonical quiet NaN.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  const uint32_t u = __float_as_uint(f);
-  const uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-  return ((u & 0x7fffffffu) > 0x7f800000u) ? 0x7fc0u : r;
-}
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 // fp16 <-> fp32 conversions are kept apart from the neighbouring multiplies: left alone the
 // compiler folds `(_Float16)(x * s)` into a mixed-precision fma with a +0 addend, which
@@ -104,6 +100,15 @@ __device__ __forceinline__ float f16_to_f32(_Float16 h) { return opaque((float)h
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
   return (uint32_t)__builtin_bit_cast(unsigned short, f32_to_f16(f));
 }
+
+// fp32 -> bf16, round to nearest even, two elements per v_cvt_pk_bf16_f32 (the integer
+// formulation costs eight ALU operations per element, which shows in a 6-byte-per-element
+// copy).  A NaN stays a NaN; its payload bits are not specified.
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  const f32x2 v = {opaque(lo), opaque(hi)};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return f32x2_to_bf16x2_bits(f, 0.0f) & 0xffffu; }
 
 template <int DT> __device__ __forceinline__ void unpack_word(uint32_t w, float& lo, float& hi);
 template <> __device__ __forceinline__ void unpack_word<RG_F16>(uint32_t w, float& lo, float& hi) {
@@ -120,7 +125,7 @@ template <> __device__ __forceinline__ uint32_t pack_word<RG_F16>(float lo, floa
   return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
 }
 template <> __device__ __forceinline__ uint32_t pack_word<RG_BF16>(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  return f32x2_to_bf16x2_bits(lo, hi);
 }
 
 template <int DT, int E> struct Codec {   // 16-bit types
@@ -455,8 +460,8 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_tensors_kernel(Finaliz
   const int t = blockIdx.x;
   double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
   int bad = 0;
-  const int64_t end = a.tensor_chunk_begin[t + 1] * a.partials_per_chunk;
-  int64_t c = a.tensor_chunk_begin[t] * a.partials_per_chunk + threadIdx.x;
+  const int64_t end = a.tensor_chunk_begin[t + 1];
+  int64_t c = a.tensor_chunk_begin[t] + threadIdx.x;
   for (; c + 3 * kBlockThreads < end; c += 4 * kBlockThreads) {
     const double v0 = a.chunk_sumsq[c], v1 = a.chunk_sumsq[c + kBlockThreads];
     const double v2 = a.chunk_sumsq[c + 2 * kBlockThreads], v3 = a.chunk_sumsq[c + 3 * kBlockThreads];
@@ -515,6 +520,26 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_total_kernel(FinalizeA
   }
 }
 
+// After a tiled reducing pass: thread c adds chunk c's tile partials in tile order.
+__global__ __launch_bounds__(kBlockThreads) void fold_tiles_kernel(const double* __restrict__ tile_sumsq,
+                                                                   const int32_t* __restrict__ tile_bad,
+                                                                   double* __restrict__ chunk_sumsq,
+                                                                   int32_t* __restrict__ chunk_bad, int64_t n_chunks,
+                                                                   int tiles_per_chunk) {
+  const int64_t c = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+  if (c >= n_chunks) return;
+  double s = 0.0;
+  int bad = 0;
+  const double* ts = tile_sumsq + c * tiles_per_chunk;
+  const int32_t* tb = tile_bad + c * tiles_per_chunk;
+  for (int t = 0; t < tiles_per_chunk; ++t) {
+    s += ts[t];
+    bad |= tb[t];
+  }
+  chunk_sumsq[c] = s;
+  chunk_bad[c] = bad;
+}
+
 __global__ __launch_bounds__(kBlockThreads) void fill_zero_kernel(char* p, int64_t nbytes) {
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
   int64_t head = (int64_t)((16u - (unsigned)(a & 15u)) & 15u);
@@ -552,6 +577,15 @@ hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream) {
   if (a.n_tensors > 0)
     hipLaunchKernelGGL(finalize_tensors_kernel, dim3((unsigned)a.n_tensors), dim3(kBlockThreads), 0, stream, a);
   hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_fold_tiles(const double* tile_sumsq, const int32_t* tile_bad, double* chunk_sumsq, int32_t* chunk_bad,
+                             int64_t n_chunks, int tiles_per_chunk, hipStream_t stream) {
+  if (n_chunks <= 0) return hipSuccess;
+  const unsigned blocks = (unsigned)((n_chunks + kBlockThreads - 1) / kBlockThreads);
+  hipLaunchKernelGGL(fold_tiles_kernel, dim3(blocks), dim3(kBlockThreads), 0, stream, tile_sumsq, tile_bad, chunk_sumsq,
+                     chunk_bad, n_chunks, tiles_per_chunk);
   return hipGetLastError();
 }
 
