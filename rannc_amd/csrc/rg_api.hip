@@ -87,7 +87,6 @@ struct rg_plan {
   float* d_tensor_norm = nullptr;
   double* d_tensor_sq = nullptr;
   int32_t* d_tensor_bad = nullptr;
-  unsigned int* d_ticket = nullptr;
   StepResult* d_result = nullptr;
 
   // pinned host memory: two chunk-table staging buffers (pointer updates stay stream
@@ -280,7 +279,6 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   const size_t o_tnorm = carve(nt * sizeof(float));
   const size_t o_tsq = carve(nt * sizeof(double));
   const size_t o_tbad = carve(nt * sizeof(int32_t));
-  const size_t o_ticket = carve(sizeof(unsigned int));
   const size_t o_result = carve(sizeof(StepResult));
   p->dev_bytes = off;
 
@@ -300,7 +298,6 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->d_tensor_norm = reinterpret_cast<float*>(b + o_tnorm);
   p->d_tensor_sq = reinterpret_cast<double*>(b + o_tsq);
   p->d_tensor_bad = reinterpret_cast<int32_t*>(b + o_tbad);
-  p->d_ticket = reinterpret_cast<unsigned int*>(b + o_ticket);
   p->d_result = reinterpret_cast<StepResult*>(b + o_result);
 
   const size_t stage_bytes = (nc * sizeof(ChunkRec) + 255) / 256 * 256;

@@ -59,12 +59,15 @@ template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
 }
 // Stores: the pointer type promises element alignment only (what the peel guarantees beyond
 // that is a performance matter, not a correctness one).
+#ifndef RG_NT_STORES
+#define RG_NT_STORES 1
+#endif
 template <bool NT> __device__ __forceinline__ void st16(char* p, u32x4 v) {
-  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_a2*>(p));
+  if (NT && RG_NT_STORES) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_a2*>(p));
   else *reinterpret_cast<u32x4_a2*>(p) = v;
 }
 template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
-  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x2_a2*>(p));
+  if (NT && RG_NT_STORES) __builtin_nontemporal_store(v, reinterpret_cast<u32x2_a2*>(p));
   else *reinterpret_cast<u32x2_a2*>(p) = v;
 }
 
@@ -163,15 +166,6 @@ template <> __device__ __forceinline__ float round_dst<RG_BF16>(float v) {
   return bf16_bits_to_f32(f32_to_bf16_bits(v));
 }
 
-template <int DT> __device__ __forceinline__ float load1(const char* p) {
-  return *reinterpret_cast<const float*>(p);
-}
-template <> __device__ __forceinline__ float load1<RG_F16>(const char* p) {
-  return f16_to_f32(*reinterpret_cast<const _Float16*>(p));
-}
-template <> __device__ __forceinline__ float load1<RG_BF16>(const char* p) {
-  return bf16_bits_to_f32(*reinterpret_cast<const unsigned short*>(p));
-}
 template <int DT> __device__ __forceinline__ void store1(char* p, float v) {
   *reinterpret_cast<float*>(p) = v;
 }
