@@ -31,7 +31,7 @@ def _sorted(items: Dict[str, Shape]) -> NamedShapes:
 
 
 def mlp_params(layers: int = 4, width: int = 1024) -> NamedShapes:
-    """C1: ``layers`` x Linear(width, width) with biases (8 tensors, 4,198,400 elements)."""
+    """``c1_mlp``: ``layers`` x Linear(width, width) with biases (8 tensors, 4,198,400 elements)."""
     out: Dict[str, Shape] = {}
     for i in range(layers):
         out[f"layers.{i}.weight"] = (width, width)
@@ -41,8 +41,8 @@ def mlp_params(layers: int = 4, width: int = 1024) -> NamedShapes:
 
 def bert_params(layers: int, hidden: int, ffn: int, vocab: int = 30522,
                 max_pos: int = 512, type_vocab: int = 2) -> NamedShapes:
-    """BERT encoder parameter list (C2: 24/1024/4096 -> 391 tensors, ~3.35e8;
-    C3: 48/2048/8192 -> 775 tensors, ~2.48e9)."""
+    """BERT encoder parameter list (``c2_bert_large``: 24/1024/4096 -> 391 tensors, ~3.35e8;
+    ``c3_bert_enlarged``: 48/2048/8192 -> 775 tensors, ~2.48e9)."""
     out: Dict[str, Shape] = {
         "bert.embeddings.word_embeddings.weight": (vocab, hidden),
         "bert.embeddings.position_embeddings.weight": (max_pos, hidden),
@@ -79,7 +79,7 @@ def bert_enlarged_params() -> NamedShapes:
 
 
 def resnet152_params(width_mult: int = 2, split: int = 2, num_classes: int = 1000) -> NamedShapes:
-    """C4: ResNet-152 bottleneck parameter list with channel widths multiplied by
+    """``c4_resnet152x2``: ResNet-152 bottleneck parameter list with channel widths multiplied by
     ``width_mult``; every tensor is then cut along dim 0 into ``split`` equal
     parts (the share layout of a x``split`` output-channel split), which gives
     934 tensors / ~2.3e8 elements with BN vectors of 64..2048 elements for the
@@ -119,7 +119,7 @@ def resnet152_params(width_mult: int = 2, split: int = 2, num_classes: int = 100
 
 def zero_segment_sizes(n_segments: int = 4096, total: int = 10_000_000_000,
                        lo: int = 1 << 10, hi: int = 1 << 26, seed: int = 0) -> List[int]:
-    """C5: ``n_segments`` parameter sizes, log-uniform in [lo, hi], rescaled so the
+    """ZeRO flat-buffer configuration: ``n_segments`` parameter sizes, log-uniform in [lo, hi], rescaled so the
     sum is close to ``total`` and forced odd (so every running offset in the flat
     buffer alternates parity and nothing is 16-byte aligned by luck)."""
     rng = np.random.default_rng(seed)

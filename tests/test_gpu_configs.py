@@ -1,6 +1,6 @@
 """The five benchmark configurations on the GPU.
 
-* against the CPU oracle at sizes it finishes in seconds (C1 in full, the others with every
+* against the CPU oracle at sizes it finishes in seconds (``c1_mlp`` in full, the others with every
   tensor's dim 0 scaled down, same tensor list and dtypes);
 * at full size through properties that do not depend on size: the unscale by a power of two is
   an exact exponent shift, so the packed bucket must equal ``(x.float() * inv) * coef``
