@@ -24,6 +24,26 @@ HIPCC_FLAGS = [
 ]
 
 
+def build_pybind(verbose: bool = True) -> str:
+    """Compile rannc_amd/_ranncgrad (pybind11 entry points over the C ABI; host code only)."""
+    import sysconfig
+
+    import pybind11
+
+    out = os.path.join(HERE, "_ranncgrad" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
+           "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"], "-I", os.path.join(ROOT, "include"),
+           os.path.join(HERE, "csrc", "rg_pybind.cpp"), "-o", out + ".tmp",
+           "-L", HERE, "-l:" + LIB_NAME, "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"pybind11 build failed ({proc.returncode}):\n{proc.stdout}")
+    os.replace(out + ".tmp", out)
+    return out
+
+
 def build(verbose: bool = True) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     srcs = [os.path.join(HERE, "csrc", s) for s in SOURCES]
@@ -43,4 +63,5 @@ def build(verbose: bool = True) -> str:
 
 if __name__ == "__main__":
     build()
+    build_pybind()
     sys.exit(0)

@@ -1,0 +1,219 @@
+// pybind11 entry points over the C ABI of libranncgrad that accept PyTorch-ROCm tensors
+// directly (module rannc_amd._ranncgrad).  The reference's boundary for this path is a
+// pybind11 module too (PYBIND11_MODULE(_pyrannc), src/main.cpp:30); like it, this layer only
+// converts arguments (tensor -> pointer, element count, dtype code, current stream) and
+// translates status codes into Python exceptions: std::invalid_argument -> ValueError,
+// std::runtime_error -> RuntimeError.  No torch headers are needed: tensors are inspected
+// through their Python attributes.
+#include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "ranncgrad.h"
+
+namespace py = pybind11;
+
+namespace {
+
+void check(int rc) {
+  if (rc == RG_OK) return;
+  const std::string msg = rg_last_error();
+  if (rc == RG_EINVAL || rc == RG_EALIGN) throw std::invalid_argument(msg);
+  if (rc == RG_ENOMEM) throw std::bad_alloc();
+  throw std::runtime_error(msg);
+}
+
+int dtype_code(const py::handle& tensor) {
+  const std::string name = py::str(tensor.attr("dtype"));
+  if (name == "torch.float32") return RG_F32;
+  if (name == "torch.float16") return RG_F16;
+  if (name == "torch.bfloat16") return RG_BF16;
+  throw std::invalid_argument("unsupported dtype " + name + ": expected float32, float16 or bfloat16");
+}
+
+struct Ref {
+  void* ptr = nullptr;
+  int64_t numel = 0;
+  int dtype = -1;
+  int device = -1;
+  bool defined = false;
+};
+
+Ref tensor_ref(const py::handle& t, const char* what, size_t i) {
+  Ref r;
+  if (t.is_none()) return r;
+  if (!t.attr("is_cuda").cast<bool>())
+    throw std::invalid_argument(std::string(what) + "[" + std::to_string(i) + "] is not on a GPU");
+  if (!t.attr("is_contiguous")().cast<bool>())
+    throw std::invalid_argument(std::string(what) + "[" + std::to_string(i) + "] is not contiguous");
+  r.defined = true;
+  r.numel = t.attr("numel")().cast<int64_t>();
+  r.dtype = dtype_code(t);
+  r.device = t.attr("device").attr("index").cast<int>();
+  r.ptr = r.numel ? reinterpret_cast<void*>(t.attr("data_ptr")().cast<uintptr_t>()) : nullptr;
+  return r;
+}
+
+void* current_stream(int device) {
+  py::object torch = py::module_::import("torch");
+  py::object s = torch.attr("cuda").attr("current_stream")(device);
+  return reinterpret_cast<void*>(s.attr("cuda_stream").cast<uintptr_t>());
+}
+
+struct Tables {
+  std::vector<const void*> src;
+  std::vector<void*> dst;
+  std::vector<int64_t> numel;
+  std::vector<int> sdt, ddt;
+  int device = -1;
+};
+
+Tables make_tables(const py::sequence& srcs, const py::object& dsts_obj) {
+  Tables t;
+  const size_t n = py::len(srcs);
+  const bool has_dst = !dsts_obj.is_none();
+  py::sequence dsts = has_dst ? dsts_obj.cast<py::sequence>() : py::sequence(py::list());
+  if (has_dst && py::len(dsts) != n) throw std::invalid_argument("srcs and dsts differ in length");
+  for (size_t i = 0; i < n; ++i) {
+    const Ref s = tensor_ref(srcs[i], "src", i);
+    const Ref d = has_dst ? tensor_ref(dsts[i], "dst", i) : Ref();
+    if (!s.defined && !d.defined) throw std::invalid_argument("pair " + std::to_string(i) + " has neither source nor destination");
+    if (s.defined && d.defined && s.numel != d.numel)
+      throw std::invalid_argument("pair " + std::to_string(i) + ": source and destination differ in element count");
+    const Ref& any = s.defined ? s : d;
+    if (t.device < 0) t.device = any.device;
+    if ((s.defined && s.device != t.device) || (d.defined && d.device != t.device))
+      throw std::invalid_argument("pair " + std::to_string(i) + " is on another device");
+    t.src.push_back(s.ptr);
+    t.dst.push_back(d.ptr);
+    t.numel.push_back(any.numel);
+    t.sdt.push_back(s.defined ? s.dtype : d.dtype);
+    t.ddt.push_back(d.defined ? d.dtype : s.dtype);
+  }
+  if (t.device < 0) t.device = 0;
+  return t;
+}
+
+class Plan {
+ public:
+  Plan(const py::sequence& srcs, const py::object& dsts, int64_t chunk_elems) : keep_src_(srcs), keep_dst_(dsts) {
+    const Tables t = make_tables(srcs, dsts);
+    device_ = t.device;
+    n_ = (int)t.numel.size();
+    check(rg_plan_create(&plan_, device_, n_, t.src.data(), t.dst.data(), t.numel.data(), t.sdt.data(), t.ddt.data(),
+                         chunk_elems));
+  }
+  ~Plan() { close(); }
+  Plan(const Plan&) = delete;
+  Plan& operator=(const Plan&) = delete;
+
+  void close() {
+    if (plan_ != nullptr) {
+      rg_plan_destroy(plan_);
+      plan_ = nullptr;
+    }
+  }
+  void update(const py::sequence& srcs, const py::object& dsts) {
+    const Tables t = make_tables(srcs, dsts);
+    if ((int)t.numel.size() != n_) throw std::invalid_argument("update: the number of tensors changed");
+    check(rg_plan_update_pointers(handle(), t.src.data(), dsts.is_none() ? nullptr : t.dst.data(), current_stream(device_)));
+    keep_src_ = srcs;
+    if (!dsts.is_none()) keep_dst_ = dsts;
+  }
+  void fused_step(float inv_scale, float max_norm, int flags) { check(rg_fused_step(handle(), inv_scale, max_norm, flags, current_stream(device_))); }
+  void step_begin(float inv_scale) { check(rg_step_begin(handle(), inv_scale, current_stream(device_))); }
+  void step_finish(float max_norm, int flags) { check(rg_step_finish(handle(), max_norm, flags, current_stream(device_))); }
+  void unscale_pack(float inv_scale) { check(rg_unscale_pack(handle(), inv_scale, current_stream(device_))); }
+  void grad_norm() { check(rg_grad_norm(handle(), current_stream(device_))); }
+  void scale_cast(float scale) { check(rg_scale_cast(handle(), scale, current_stream(device_))); }
+  void zero() { check(rg_zero(handle(), current_stream(device_))); }
+  py::dict result() {
+    rg_step_result r;
+    check(rg_read_result(handle(), &r, current_stream(device_)));
+    py::dict d;
+    d["norm"] = r.norm;
+    d["coef"] = r.coef;
+    d["overflow"] = r.overflow;
+    d["clipped"] = r.clipped;
+    d["skipped"] = r.skipped;
+    return d;
+  }
+  std::vector<float> tensor_norms() {
+    std::vector<float> out((size_t)(n_ > 0 ? n_ : 1));
+    check(rg_read_tensor_norms(handle(), out.data(), current_stream(device_)));
+    out.resize((size_t)n_);
+    return out;
+  }
+  int64_t num_chunks() const { return rg_plan_num_chunks(plan_); }
+  int64_t chunk_elems() const { return rg_plan_chunk_elems(plan_); }
+  int64_t total_numel() const { return rg_plan_total_numel(plan_); }
+  int num_tensors() const { return n_; }
+
+ private:
+  rg_plan* handle() {
+    if (plan_ == nullptr) throw std::runtime_error("the plan is closed");
+    return plan_;
+  }
+  rg_plan* plan_ = nullptr;
+  int device_ = 0;
+  int n_ = 0;
+  py::object keep_src_, keep_dst_;  // the table points into these tensors
+};
+
+void copy_cast(const py::handle& dst, const py::handle& src, float scale) {
+  const Ref d = tensor_ref(dst, "dst", 0);
+  const Ref s = tensor_ref(src, "src", 0);
+  if (!d.defined) throw std::invalid_argument("copy_cast needs a destination");
+  if (s.defined && (s.numel != d.numel || s.device != d.device))
+    throw std::invalid_argument("copy_cast: source and destination differ in element count or device");
+  check(rg_scale_cast_single(s.ptr, d.ptr, d.numel, s.defined ? s.dtype : d.dtype, d.dtype, scale, d.device,
+                             current_stream(d.device)));
+}
+
+}  // namespace
+
+PYBIND11_MODULE(_ranncgrad, m) {
+  m.doc() = "pybind11 entry points of libranncgrad (per-step parameter/gradient path, MI355X)";
+  m.attr("RG_F32") = (int)RG_F32;
+  m.attr("RG_F16") = (int)RG_F16;
+  m.attr("RG_BF16") = (int)RG_BF16;
+  m.attr("STEP_DEFAULT") = (int)RG_STEP_DEFAULT;
+  m.attr("STEP_WRITE_ON_OVERFLOW") = (int)RG_STEP_WRITE_ON_OVERFLOW;
+  m.attr("STEP_IGNORE_OVERFLOW") = (int)RG_STEP_IGNORE_OVERFLOW;
+  m.def("version", &rg_version);
+  m.def("aligned_numel", [](int64_t numel, int elem_size, int split) {
+    const int64_t r = rg_aligned_numel(numel, elem_size, split);
+    if (r < 0) throw std::invalid_argument(rg_last_error());
+    return r;
+  });
+  m.def("segment_layout", [](int64_t numel, int elem_size, int nranks) {
+    if (nranks < 1) throw std::invalid_argument("nranks must be >= 1");
+    int64_t aligned = 0, seg = 0;
+    std::vector<int64_t> offs((size_t)nranks), srcs((size_t)nranks);
+    check(rg_segment_layout(numel, elem_size, nranks, &aligned, &seg, offs.data(), srcs.data()));
+    return py::make_tuple(aligned, seg, offs, srcs);
+  });
+  m.def("copy_cast", &copy_cast, py::arg("dst"), py::arg("src"), py::arg("scale") = 1.0f,
+        "dst.copy_(src) with dtype conversion and optional scale for one pair of tensors; src=None stores zeros");
+  py::class_<Plan>(m, "Plan")
+      .def(py::init<const py::sequence&, const py::object&, int64_t>(), py::arg("srcs"), py::arg("dsts") = py::none(),
+           py::arg("chunk_elems") = 0)
+      .def("update", &Plan::update, py::arg("srcs"), py::arg("dsts") = py::none())
+      .def("fused_step", &Plan::fused_step, py::arg("inv_scale"), py::arg("max_norm"), py::arg("flags") = 0)
+      .def("step_begin", &Plan::step_begin)
+      .def("step_finish", &Plan::step_finish, py::arg("max_norm"), py::arg("flags") = 0)
+      .def("unscale_pack", &Plan::unscale_pack)
+      .def("grad_norm", &Plan::grad_norm)
+      .def("scale_cast", &Plan::scale_cast, py::arg("scale") = 1.0f)
+      .def("zero", &Plan::zero)
+      .def("result", &Plan::result)
+      .def("tensor_norms", &Plan::tensor_norms)
+      .def("close", &Plan::close)
+      .def_property_readonly("num_chunks", &Plan::num_chunks)
+      .def_property_readonly("chunk_elems", &Plan::chunk_elems)
+      .def_property_readonly("total_numel", &Plan::total_numel)
+      .def_property_readonly("num_tensors", &Plan::num_tensors);
+}

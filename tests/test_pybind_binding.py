@@ -1,0 +1,71 @@
+"""The pybind11 entry points (rannc_amd._ranncgrad) over the same C ABI: they take PyTorch-ROCm
+tensors directly, give the same results as the ctypes path and translate errors the way the
+reference's pybind module does (ValueError / RuntimeError)."""
+import math
+
+import pytest
+import torch
+
+from oracle import gradpath as oracle
+from rannc_amd import _lib, _ranncgrad
+from tests.helpers import assert_bits_equal
+
+
+def test_layout_and_constants_match_the_c_abi():
+    assert _ranncgrad.version() == _lib.lib.rg_version()
+    assert (_ranncgrad.RG_F32, _ranncgrad.RG_F16, _ranncgrad.RG_BF16) == (_lib.RG_F32, _lib.RG_F16, _lib.RG_BF16)
+    for numel, es, r in [(1000, 2, 8), (100, 2, 8), (7, 4, 3), (0, 4, 2)]:
+        assert tuple(_ranncgrad.segment_layout(numel, es, r)) == _lib.segment_layout(numel, es, r)
+        assert _ranncgrad.aligned_numel(numel, es, r) == oracle.calc_aligned_num_elems(numel, es, r)
+
+
+def test_errors_are_python_exceptions():
+    with pytest.raises(ValueError):
+        _ranncgrad.aligned_numel(1, 3, 1)
+    with pytest.raises(ValueError):
+        _ranncgrad.segment_layout(10, 4, 0)
+    with pytest.raises(ValueError, match="GPU"):
+        _ranncgrad.Plan([torch.zeros(4)], [torch.zeros(4)])
+    with pytest.raises(ValueError, match="GPU"):
+        _ranncgrad.copy_cast(torch.zeros(4), torch.zeros(4))
+
+
+@pytest.mark.gpu
+def test_fused_step_through_pybind_matches_oracle_and_ctypes():
+    from rannc_amd.multi_tensor import TensorPlan
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(5)
+    cpu = [(torch.randn(s, generator=g) * 1e-2 * 65536).to(torch.bfloat16) for s in [(70001,), (33,), (4096,), (0,)]]
+    srcs = [t.to(dev) for t in cpu]
+    out_a = [torch.zeros(t.shape, device=dev) for t in cpu]
+    out_b = [torch.zeros(t.shape, device=dev) for t in cpu]
+    pa = _ranncgrad.Plan(srcs, out_a)
+    pa.fused_step(2.0 ** -16, 0.25)
+    ra = pa.result()
+    pb = TensorPlan(srcs, out_b)
+    pb.fused_step(2.0 ** -16, 0.25)
+    rb = pb.result()
+    assert (ra["norm"], ra["coef"], ra["overflow"], ra["clipped"]) == (rb.norm, rb.coef, rb.overflow, rb.clipped)
+    assert pa.tensor_norms() == pb.tensor_norms() and pa.num_tensors == 4 and pa.total_numel == pb.plan.total_numel
+    want = oracle.fused_step(cpu, ["f32"] * 4, 2.0 ** -16, 0.25)
+    assert math.isclose(ra["norm"], want.norm, rel_tol=1e-6) and math.isclose(ra["coef"], want.coef, rel_tol=1e-6)
+    for a, b in zip(out_a, out_b):
+        assert_bits_equal(a.cpu(), b.cpu(), "pybind vs ctypes")
+    # the other operations and the plan-free copy
+    pa.unscale_pack(2.0 ** -16)
+    un, _ = oracle.unscale_and_check(cpu, 2.0 ** -16)
+    for a, w in zip(out_a, un):
+        assert_bits_equal(a.cpu(), w, "unscale_pack")
+    pa.zero()
+    torch.cuda.synchronize()
+    assert all(bool((a == 0).all()) for a in out_a)
+    half = torch.zeros(70001, dtype=torch.float16, device=dev)
+    _ranncgrad.copy_cast(half, srcs[0])
+    assert_bits_equal(half.cpu(), cpu[0].to(torch.float16), "copy_cast")
+    with pytest.raises(ValueError, match="contiguous"):
+        _ranncgrad.Plan([torch.zeros(4, 4, device=dev).t()], [torch.zeros(4, 4, device=dev)])
+    with pytest.raises(ValueError, match="dtype"):
+        _ranncgrad.Plan([torch.zeros(4, dtype=torch.float64, device=dev)], None)
+    pa.close()
+    with pytest.raises(RuntimeError, match="closed"):
+        pa.grad_norm()
