@@ -146,6 +146,18 @@ int rg_step_finish(rg_plan* plan, float max_norm, int flags, void* stream);
  * clip.  Apex multi_tensor_scale semantics (LossScaler.unscale). */
 int rg_unscale_pack(rg_plan* plan, float inv_scale, void* stream);
 
+/* Accumulating forms, for gradient accumulation over several backward passes:
+ *   rg_accumulate:          dst = round_dst(float(dst) + float(src) * scale)
+ *   rg_unscale_accumulate:  the same with scale = inv_scale, plus the inf/NaN flag of the sources
+ *                           and the norm of the RESULT, as rg_unscale_pack reports them.
+ * The product is rounded to fp32 before the sum (two roundings, `master.add_(model.float() *
+ * inv_scale)`).  This is Apex's unscale_with_stashed / multi_tensor_axpby (external to the
+ * reference; whether Apex's kernel contracts the two operations into one fma is not visible
+ * from the reference tree, so bit parity with Apex is not claimed for this entry point).
+ * Missing sources (NULL) add nothing.  dst must differ from src. */
+int rg_accumulate(rg_plan* plan, float scale, void* stream);
+int rg_unscale_accumulate(rg_plan* plan, float inv_scale, void* stream);
+
 /* Read-only: per-tensor and global L2 norm of the SOURCE tensors and their inf/NaN flag.
  * ParamStorage::calcGradGlobalL2Norm, src/comp/ParamStorage.cpp:747-819
  * (RaNNCModule.calc_grad_norm, src/main.cpp:344-345). */

@@ -416,3 +416,25 @@ def reference_step_cpu(model_grads: Sequence[torch.Tensor], master_grad_views: S
         for v in master_grad_views:
             v.mul_(coef)
     return 0, norm, coef
+
+
+# --------------------------------------------------------------------------- accumulation
+
+def unscale_accumulate(master_grads: Sequence[torch.Tensor], model_grads: Sequence[Optional[torch.Tensor]],
+                       inv_scale: float) -> int:
+    """Gradient accumulation under amp (Apex ``unscale_with_stashed``, external):
+    ``master_grad += float(model_grad) * inv_scale`` in place, the product rounded to fp32 before
+    the sum, the sum rounded to the master's dtype; returns the inf/NaN flag of the model grads.
+    Whether Apex's kernel fuses the two operations is not visible from the reference tree:
+    parity unpinned against Apex; pinned here against float64 arithmetic (the two roundings are
+    reproduced by numpy in the test)."""
+    scale = torch.tensor(inv_scale, dtype=torch.float32)
+    overflow = 0
+    for m, g in zip(master_grads, model_grads):
+        if g is None:
+            continue
+        gf = g.to(torch.float32)
+        if g.numel() and not bool(torch.isfinite(gf).all()):
+            overflow = 1
+        m.copy_((m.to(torch.float32) + gf * scale).to(m.dtype))
+    return overflow

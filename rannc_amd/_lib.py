@@ -47,6 +47,8 @@ SIGNATURES = {
     "rg_step_begin": (_i, [_vp, _f, _vp]),
     "rg_step_finish": (_i, [_vp, _f, _i, _vp]),
     "rg_unscale_pack": (_i, [_vp, _f, _vp]),
+    "rg_accumulate": (_i, [_vp, _f, _vp]),
+    "rg_unscale_accumulate": (_i, [_vp, _f, _vp]),
     "rg_grad_norm": (_i, [_vp, _vp]),
     "rg_scale_cast": (_i, [_vp, _f, _vp]),
     "rg_scale_cast_single": (_i, [_vp, _vp, _i64, _i, _i, _f, _i, _vp]),
@@ -68,7 +70,7 @@ class RanncGradError(RuntimeError):
 def _load() -> C.CDLL:
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m rannc_amd.build` "
+            f"{LIB_PATH} is missing: build it with `python rannc_amd/build.py` "
             "(there is no fallback path)")
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
@@ -192,6 +194,12 @@ class Plan:
 
     def unscale_pack(self, inv_scale: float, stream: int = 0) -> None:
         check(lib.rg_unscale_pack(self._handle, inv_scale, _vp(stream)))
+
+    def accumulate(self, scale: float = 1.0, stream: int = 0) -> None:
+        check(lib.rg_accumulate(self._handle, scale, _vp(stream)))
+
+    def unscale_accumulate(self, inv_scale: float, stream: int = 0) -> None:
+        check(lib.rg_unscale_accumulate(self._handle, inv_scale, _vp(stream)))
 
     def grad_norm(self, stream: int = 0) -> None:
         check(lib.rg_grad_norm(self._handle, _vp(stream)))

@@ -16,8 +16,10 @@ Two layers live here:
 The dynamic loss-scale schedule (halve on overflow, double after ``scale_window`` clean
 steps) is this project's own statement of the usual policy; Apex's is not in the tree.
 
-Gradient accumulation over several ``scale_loss`` contexts is not supported: master
-gradients are overwritten, not accumulated, by each unscale.
+Gradient accumulation follows PyTorch's convention: a master gradient that is still defined
+when a ``scale_loss`` context exits (no ``zero_grad`` since the last one) is accumulated into
+(``master_grad += float(model_grad) * inv_scale``, Apex's ``unscale_with_stashed``); one that
+is ``None`` is overwritten.
 """
 from __future__ import annotations
 
@@ -84,10 +86,12 @@ class LossScaler:
     def clear_overflow_state(self) -> None:
         self._has_overflow = False
 
-    def unscale(self, stash: _AmpStash, model_grads: List[torch.Tensor], master_grads: List[torch.Tensor]) -> None:
+    def unscale(self, stash: _AmpStash, model_grads: List[torch.Tensor], master_grads: List[torch.Tensor],
+                accumulate: bool = False) -> None:
         """``master_grad = float(model_grad) * (1 / scale)`` for every pair in one launch, with the
         inf/NaN flag and - for free - the gradient norm.  In fused mode only the read pass runs
-        here; the values are written by ``finish_unscale``."""
+        here; the values are written by ``finish_unscale``.  ``accumulate`` adds to the master
+        gradients instead of overwriting them (always eager)."""
         key = tuple((g.data_ptr(), g.numel(), g.dtype, m.data_ptr(), m.dtype) for g, m in zip(model_grads, master_grads))
         if stash.unscale_plan is None or stash.unscale_key != key:
             if stash.unscale_plan is not None:
@@ -96,7 +100,9 @@ class LossScaler:
             stash.unscale_key = key
         inv = 1.0 / self._loss_scale
         with torch.no_grad():
-            if stash.fused:
+            if accumulate:
+                stash.unscale_plan.unscale_accumulate(inv)
+            elif stash.fused:
                 stash.unscale_plan.step_begin(inv)
                 stash.pending_finish = True
             else:
@@ -249,16 +255,28 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
         stash.master_grad_bucket = torch.empty(lens[_lib.RG_F32], dtype=torch.float32, device=masters[0].device)
         stash.master_grad_views = [stash.master_grad_bucket.narrow(0, o, m.numel()).view(m.shape)
                                    for o, m in zip(offs, masters)]
+    fresh, live = [], []
     for i, (p, m) in enumerate(zip(stash.all_fp16_params, stash.all_fp32_from_fp16_params)):
         if p.grad is None:
             continue
+        (fresh if m.grad is None else live).append(i)
+    accumulate = bool(live)
+    if accumulate:
+        finish_unscale(optimizer)                 # a deferred write must land before it is added to
+        from ..multi_tensor import fill_zero_
+        for i in fresh:                           # mixed case: start the missing ones from zero
+            m = stash.all_fp32_from_fp16_params[i]
+            m.grad = stash.master_grad_views[i]
+            fill_zero_(m.grad.view(-1)) if m.grad.is_contiguous() else m.grad.zero_()
+    for i in sorted(fresh + live):
+        p, m = stash.all_fp16_params[i], stash.all_fp32_from_fp16_params[i]
         if m.grad is None:
             m.grad = stash.master_grad_views[i]
         model_grads.append(p.grad)
         master_grads.append(m.grad)
     scaler.clear_overflow_state()
     if model_grads:
-        scaler.unscale(stash, model_grads, master_grads)
+        scaler.unscale(stash, model_grads, master_grads, accumulate=accumulate)
     # fp32 parameters keep their own .grad; it carries the loss scale too
     fp32_grads = [p.grad for p in stash.all_fp32_from_fp32_params if p.grad is not None]
     if fp32_grads:

@@ -1,6 +1,7 @@
 """Build libranncgrad.so (the HIP kernel library) in-tree for gfx950.
 
-Run as ``python -m rannc_amd.build``; ``__graft_entry__.build()`` calls :func:`build`.
+Run as ``python rannc_amd/build.py`` (by path, so that the package - which loads the library on
+import - is not imported first); ``__graft_entry__.build()`` calls :func:`build` the same way.
 """
 from __future__ import annotations
 

@@ -542,6 +542,56 @@ RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   return RG_OK;
 }
 
+static int check_not_in_place(const rg_plan* p, const char* op) {
+  for (int i = 0; i < p->n_tensors; ++i) {
+    const TensorDesc& t = p->host_tensors[(size_t)i];
+    if (t.numel > 0 && t.src != nullptr && t.src == t.dst) {
+      set_error("%s: tensor %d accumulates into itself", op, i);
+      return RG_EINVAL;
+    }
+  }
+  return RG_OK;
+}
+
+RG_API int rg_accumulate(rg_plan* p, float scale, void* stream) {
+  int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_accumulate");
+  if (rc == RG_OK) rc = check_not_in_place(p, "rg_accumulate");
+  if (rc != RG_OK) return rc;
+  DeviceGuard guard(p->device);
+  PassArgs a = pass_args(p, scale);
+  split_for_write(p, a);
+  RG_HIP(launch_pass(kModeWrite | kModeAccumulate, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
+  return RG_OK;
+}
+
+RG_API int rg_unscale_accumulate(rg_plan* p, float inv_scale, void* stream) {
+  int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_unscale_accumulate");
+  if (rc == RG_OK) rc = check_not_in_place(p, "rg_unscale_accumulate");
+  if (rc != RG_OK) return rc;
+  if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
+    set_error("rg_unscale_accumulate: inv_scale must be a non-zero number");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  PassArgs a = pass_args(p, inv_scale);
+  split_for_write(p, a);
+  if (a.tiles_per_chunk > 1 && a.tile_elems * 2 <= p->chunk_elems) {
+    a.tile_elems *= 2;
+    a.tiles_per_chunk = (int32_t)((p->chunk_elems + a.tile_elems - 1) / a.tile_elems);
+  }
+  if (a.tiles_per_chunk > 1) {
+    a.chunk_sumsq = p->d_tile_sumsq;
+    a.chunk_bad = p->d_tile_bad;
+  }
+  RG_HIP(launch_pass(kModeReduce | kModeWrite | kModeAccumulate, a, p->streaming, s));
+  if (a.tiles_per_chunk > 1)
+    RG_HIP(launch_fold_tiles(p->d_tile_sumsq, p->d_tile_bad, p->d_chunk_sumsq, p->d_chunk_bad, p->n_chunks,
+                             a.tiles_per_chunk, s));
+  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
+  return RG_OK;
+}
+
 RG_API int rg_grad_norm(rg_plan* p, void* stream) {
   const int rc = check_plan(p, kNeedSrc, "rg_grad_norm");
   if (rc != RG_OK) return rc;

@@ -86,7 +86,7 @@ constexpr int64_t kMaxChunkElems = 1 << 20;
 constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan
 
 // Pass selection for the chunk kernel.
-enum : int { kModeReduce = 1, kModeWrite = 2 };
+enum : int { kModeReduce = 1, kModeWrite = 2, kModeAccumulate = 4 };  // accumulate: dst = round(dst + x * scale)
 
 struct PassArgs {
   const ChunkRec* chunks;        // [n_chunks]; null = one tensor described by `single`

@@ -19,6 +19,8 @@
 //
 // The work is purely bandwidth bound (a few ALU ops per element): no LDS staging and no
 // MFMA.  LDS is used only for the 4-wavefront combine of the partial sums.
+#include <type_traits>
+
 #include "rg_internal.h"
 
 namespace rg {
@@ -190,14 +192,14 @@ template <> __device__ __forceinline__ bool nonfinite_at<RG_BF16>(const char* p)
 // coef is 1 when nothing is clipped: v * 1 is v bit for bit, so no branch is needed.
 // The two multiplies are never fused or reassociated (the file is built with
 // -ffp-contract=off), so the result matches `x.float() * inv_scale` then `mul_(coef)`.
-template <int S, int D, int MODE, bool NT>
+template <int S, int D, int MODE, bool NT, int T = PassThreads<MODE>::value>
 __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len, float scale, float coef,
                                               bool raw_copy, float (&acc)[8]) {
-  constexpr int T = PassThreads<MODE>::value;
   constexpr int SS = ElemSize<S>::value;
   constexpr int DS = ElemSize<D>::value;
   constexpr bool kWrite = (MODE & kModeWrite) != 0;
   constexpr bool kReduce = (MODE & kModeReduce) != 0;
+  constexpr bool kAcc = (MODE & kModeAccumulate) != 0;   // dst = round_dst(float(dst) + x * scale)
   constexpr int E = (SS == 4 || (kWrite && DS == 4)) ? 4 : 8;   // elements per lane per instruction
   constexpr int kPerThread = kWrite ? kWriteElemsPerThread : kReduceElemsPerThread;
   constexpr int U = kPerThread >= E ? kPerThread / E : 1;      // instructions in flight per lane
@@ -228,7 +230,15 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
       if (S == RG_F32) x = __uint_as_float(raw);
       else if (S == RG_F16) x = f16_to_f32(__builtin_bit_cast(_Float16, (unsigned short)raw));
       else x = bf16_bits_to_f32(raw);
-      const float v = round_dst<D>(x * scale);
+      float t = x * scale;
+      if (kAcc) {
+        float old;
+        if (D == RG_F32) old = *reinterpret_cast<const float*>(dp + (size_t)i * 4);
+        else if (D == RG_F16) old = f16_to_f32(*reinterpret_cast<const _Float16*>(dp + (size_t)i * 2));
+        else old = bf16_bits_to_f32(*reinterpret_cast<const unsigned short*>(dp + (size_t)i * 2));
+        t = opaque(t) + old;
+      }
+      const float v = round_dst<D>(t);
       if (kReduce) acc[0] = __builtin_fmaf(v, v, acc[0]);
       if (kWrite) store1<D>(dp + (size_t)i * DS, v * coef);
     }
@@ -244,7 +254,10 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
 
   // All U loads of an iteration are issued back to back with no branch between them, so
   // they are all in flight together.  `valid` only guards what is accumulated and stored.
-  auto consume = [&](const Raw<S, E>& in, int e, bool valid) {
+  // previous destination values, only when accumulating (the type does not exist otherwise)
+  struct Nothing {};
+  using Old = std::conditional_t<kAcc, Raw<kAcc ? D : S, E>, Nothing>;
+  auto consume = [&](const Raw<S, E>& in, const Old* old, int e, bool valid) {
     bool copied = false;
     if constexpr (S == D && kWrite) {
       if (raw_copy) {
@@ -255,9 +268,13 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
     if (!copied) {
       float f[E];
       Codec<S, E>::unpack(in, f);
+      float o[E];
+      if constexpr (kAcc) Codec<D, E>::unpack(*old, o);
 #pragma unroll
       for (int j = 0; j < E; ++j) {
-        float v = round_dst<D>(f[j] * scale);
+        float t = f[j] * scale;
+        if constexpr (kAcc) t = opaque(t) + o[j];   // product rounded first, then the sum
+        float v = round_dst<D>(t);
         if (kReduce) {
           const float q = valid ? v : 0.0f;
           acc[j & 7] = __builtin_fmaf(q, q, acc[j & 7]);
@@ -273,24 +290,31 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   int base = 0;
   for (; base + kIter <= nbody; base += kIter) {
     Raw<S, E> in[U];
+    Old old[kAcc ? U : 1];
 #pragma unroll
     for (int u = 0; u < U; ++u) in[u] = Mem<S, E, NT>::load(sb + (size_t)(base + (u * T + tid) * E) * SS);
+    if constexpr (kAcc) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) consume(in[u], base + (u * T + tid) * E, true);
+      for (int u = 0; u < U; ++u) old[u] = Mem<D, E, NT>::load(db + (size_t)(base + (u * T + tid) * E) * DS);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) consume(in[u], &old[kAcc ? u : 0], base + (u * T + tid) * E, true);
   }
   if (base < nbody) {
     // Last, partial iteration: lanes past the end re-read the final vector (an address that
     // is certainly valid) so the loads stay unconditional, and are masked afterwards.
     Raw<S, E> in[U];
+    Old old[kAcc ? U : 1];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int e = base + (u * T + tid) * E;
       in[u] = Mem<S, E, NT>::load(sb + (size_t)(e < nbody ? e : nbody - E) * SS);
+      if constexpr (kAcc) old[u] = Mem<D, E, NT>::load(db + (size_t)(e < nbody ? e : nbody - E) * DS);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int e = base + (u * T + tid) * E;
-      consume(in[u], e, e < nbody);
+      consume(in[u], &old[kAcc ? u : 0], e, e < nbody);
     }
   }
 
@@ -375,11 +399,20 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
   char* dp = reinterpret_cast<char*>(rec.dst) + (size_t)start * (rec.dst_dtype == RG_F32 ? 4 : 2);
   const int src_kind = rec.src_dtype;
   const int dst_kind = a.norm_of_source ? rec.src_dtype : rec.dst_dtype;
-  const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale == 1.0f;
+  const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale == 1.0f;   // never when accumulating
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (sp == nullptr || a.zero_fill) {
-    if (MODE & kModeWrite) zero_range<NT, T>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
+    if constexpr ((MODE & kModeAccumulate) != 0) {
+      // Nothing to add: the destination keeps its values, which still count towards the norm.
+      if constexpr ((MODE & kModeReduce) != 0) {
+        if (dst_kind == RG_F32) process_chunk<RG_F32, RG_F32, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
+        else if (dst_kind == RG_F16) process_chunk<RG_F16, RG_F16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
+        else process_chunk<RG_BF16, RG_BF16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
+      }
+    } else if (MODE & kModeWrite) {
+      zero_range<NT, T>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
+    }
   } else {
     switch (src_kind * 3 + dst_kind) {
       case RG_F32 * 3 + RG_F32: process_chunk<RG_F32, RG_F32, MODE, NT>(sp, dp, len, a.scale, coef, raw_copy, acc); break;
@@ -562,7 +595,12 @@ hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t 
   switch (mode) {
     case kModeReduce: launch_mode<kModeReduce>(a, streaming, stream); break;
     case kModeWrite: launch_mode<kModeWrite>(a, streaming, stream); break;
-    default: launch_mode<kModeReduce | kModeWrite>(a, streaming, stream); break;
+    case kModeReduce | kModeWrite: launch_mode<kModeReduce | kModeWrite>(a, streaming, stream); break;
+    case kModeWrite | kModeAccumulate: launch_mode<kModeWrite | kModeAccumulate>(a, streaming, stream); break;
+    case kModeReduce | kModeWrite | kModeAccumulate:
+      launch_mode<kModeReduce | kModeWrite | kModeAccumulate>(a, streaming, stream);
+      break;
+    default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }

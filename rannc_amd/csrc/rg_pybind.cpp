@@ -127,6 +127,10 @@ class Plan {
   void step_begin(float inv_scale) { check(rg_step_begin(handle(), inv_scale, current_stream(device_))); }
   void step_finish(float max_norm, int flags) { check(rg_step_finish(handle(), max_norm, flags, current_stream(device_))); }
   void unscale_pack(float inv_scale) { check(rg_unscale_pack(handle(), inv_scale, current_stream(device_))); }
+  void accumulate(float scale) { check(rg_accumulate(handle(), scale, current_stream(device_))); }
+  void unscale_accumulate(float inv_scale) {
+    check(rg_unscale_accumulate(handle(), inv_scale, current_stream(device_)));
+  }
   void grad_norm() { check(rg_grad_norm(handle(), current_stream(device_))); }
   void scale_cast(float scale) { check(rg_scale_cast(handle(), scale, current_stream(device_))); }
   void zero() { check(rg_zero(handle(), current_stream(device_))); }
@@ -206,6 +210,8 @@ PYBIND11_MODULE(_ranncgrad, m) {
       .def("step_begin", &Plan::step_begin)
       .def("step_finish", &Plan::step_finish, py::arg("max_norm"), py::arg("flags") = 0)
       .def("unscale_pack", &Plan::unscale_pack)
+      .def("accumulate", &Plan::accumulate, py::arg("scale") = 1.0f)
+      .def("unscale_accumulate", &Plan::unscale_accumulate)
       .def("grad_norm", &Plan::grad_norm)
       .def("scale_cast", &Plan::scale_cast, py::arg("scale") = 1.0f)
       .def("zero", &Plan::zero)

@@ -131,6 +131,12 @@ class TensorPlan:
     def unscale_pack(self, inv_scale: float) -> None:
         self.plan.unscale_pack(inv_scale, self._stream())
 
+    def accumulate(self, scale: float = 1.0) -> None:
+        self.plan.accumulate(scale, self._stream())
+
+    def unscale_accumulate(self, inv_scale: float) -> None:
+        self.plan.unscale_accumulate(inv_scale, self._stream())
+
     def grad_norm(self) -> None:
         self.plan.grad_norm(self._stream())
 

@@ -293,6 +293,29 @@ def test_amp_step_matches_oracle_sequence(fused, half):
     rm.zero_grad()
 
 
+def test_amp_gradient_accumulation_adds_into_live_master_grads():
+    model = _tiny_model()
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    xs = [torch.randn(16, 32, device=DEV, dtype=torch.float16) for _ in range(3)]
+    want = None
+    for x in xs:                                             # three micro-batches, no zero_grad between
+        loss = rm(x).float().pow(2).mean()
+        with amp.scale_loss(loss, opt) as scaled:
+            scaled.backward()
+            grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
+        if want is None:
+            want, _ = oracle.unscale_and_check(grads, 1.0 / 256.0)
+        else:
+            oracle.unscale_accumulate(want, grads, 1.0 / 256.0)
+    for m, w in zip(opt._amp_stash.all_fp32_from_fp16_params, want):
+        assert_bits_equal(m.grad.cpu(), w, "accumulated master grad")
+    opt.step()
+    opt.zero_grad()
+    assert all(m.grad is None or bool((m.grad == 0).all()) for m in opt._amp_stash.all_fp32_from_fp16_params)
+
+
 def test_amp_overflow_skips_the_step_and_halves_the_scale():
     model = _tiny_model()
     opt = torch.optim.SGD(model.parameters(), lr=0.1)

@@ -220,3 +220,37 @@ def test_error_paths():
         TensorPlan([a], [a.view(torch.int32).view(torch.float32)]).plan  # same dtype in place is fine
         b16 = torch.zeros(20, dtype=torch.bfloat16, device=DEV)
         _lib.scale_cast_single(b16.data_ptr(), b16.data_ptr(), 10, _lib.RG_BF16, _lib.RG_F32, 1.0, 0, 0)
+
+
+@pytest.mark.parametrize("src_name,dst_name", [("f16", "f32"), ("bf16", "f32"), ("f32", "f32"), ("f16", "f16"), ("f32", "bf16")])
+def test_accumulate_and_unscale_accumulate(src_name, dst_name):
+    sdt, ddt = TORCH_DTYPE[src_name], TORCH_DTYPE[dst_name]
+    g = torch.Generator().manual_seed(17)
+    model = [(torch.randn(s, generator=g) * 64.0).to(sdt) for s in SHAPES]
+    master = [torch.randn(s, generator=g).to(ddt) for s in SHAPES]
+    srcs = place_in_arena(model, DEV, 1, 3)
+    dsts = place_in_arena(master, DEV, 2, 1)
+    plan_srcs = list(srcs)
+    plan_srcs[4] = None                                   # a parameter without a gradient adds nothing
+    plan = TensorPlan(plan_srcs, dsts, chunk_elems=2048)
+    want = [m.clone() for m in master]
+    model_with_hole = [None if i == 4 else x for i, x in enumerate(model)]
+    for step in range(2):                                 # accumulate twice
+        plan.unscale_accumulate(1.0 / 64.0)
+        flag = oracle.unscale_accumulate(want, model_with_hole, 1.0 / 64.0)
+        res = plan.result()
+        assert res.overflow == flag == 0
+        for d, w in zip(dsts, want):
+            assert_bits_equal(d.cpu(), w, f"unscale_accumulate step {step}")
+        assert math.isclose(res.norm, oracle.grad_global_l2_norm(want), rel_tol=1e-6)
+    plan.accumulate(0.25)                                 # plain axpy, no flag / norm
+    oracle.unscale_accumulate(want, model_with_hole, 0.25)
+    for d, w in zip(dsts, want):
+        assert_bits_equal(d.cpu(), w, "accumulate")
+    model[2][1] = float("inf")
+    srcs[2].copy_(model[2])
+    plan.unscale_accumulate(1.0 / 64.0)
+    assert plan.result().overflow == 1
+    with pytest.raises(ValueError, match="itself"):
+        TensorPlan([dsts[5]], [dsts[5]]).accumulate(1.0)
+    plan.close()

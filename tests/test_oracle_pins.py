@@ -297,3 +297,23 @@ def test_patched_update_scale_cases():
     # the minimum wins even when the local scale is smaller
     s = oracle.LossScalerState(loss_scale=128.0)
     assert oracle.patched_update_scale(s, False, other_flags=[1], other_scales=[512]) is True and s.loss_scale == 128
+
+
+# ----------------------------------------------------------------------------- accumulation
+
+def test_unscale_accumulate_is_two_roundings():
+    g = torch.Generator().manual_seed(8)
+    master = torch.randn(3000, generator=g)
+    model = (torch.randn(3000, generator=g) * 100).to(torch.float16)
+    want = (master.numpy().astype(np.float32)
+            + (model.numpy().astype(np.float32) * np.float32(0.37)).astype(np.float32)).astype(np.float32)
+    m = master.clone()
+    assert oracle.unscale_accumulate([m, torch.zeros(2)], [model, None], 0.37) == 0
+    assert np.array_equal(f32_bits(m), want.view(np.uint32))
+    # exact case: accumulating x/2 twice onto zero gives x
+    z = torch.zeros(3000)
+    oracle.unscale_accumulate([z], [model], 0.5)
+    oracle.unscale_accumulate([z], [model], 0.5)
+    assert torch.equal(z, model.float())
+    model[5] = float("nan")
+    assert oracle.unscale_accumulate([master.clone()], [model], 0.5) == 1
