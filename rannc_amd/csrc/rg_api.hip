@@ -5,6 +5,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <new>
 #include <vector>
 
@@ -71,9 +72,12 @@ struct rg_plan {
   int64_t n_chunks = 0;
   bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
   int64_t write_tile_elems = kWriteTileElems;
+  int xcd_reduce = 64;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
+  int xcd_write = 0;
   float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
   std::vector<TensorDesc> host_tensors;
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
+  bool dst_heads = false;            // some destination starts off a 128-byte boundary
 
   // one device allocation, carved up
   char* dev_base = nullptr;
@@ -114,18 +118,32 @@ static int check_pointer(const void* p, int esz, const char* which, int i) {
   return RG_OK;
 }
 
-// Writes the chunk records of every tensor into `out` ([n_chunks]).
-static void fill_chunk_records(const rg_plan* p, ChunkRec* out) {
+// Elements of a tensor before the first 128-byte boundary of the side its passes write
+// (the destination; the source of a plan without destinations).
+static int64_t tensor_head(const void* src, const void* dst, int ss, int ds) {
+  if (dst != nullptr) return head_elems(reinterpret_cast<uintptr_t>(dst), kWriteAlignBytes, (unsigned)ds);
+  return head_elems(reinterpret_cast<uintptr_t>(src), kAlignBytes, (unsigned)ss);
+}
+
+// Writes the chunk records of every tensor into `out` ([n_chunks]).  Chunk j of a tensor
+// covers elements [j ? head + j*C : 0, head + (j+1)*C), clipped to the tensor: every chunk but
+// the first starts on an aligned address, the first is up to `head` elements longer, and
+// the number of chunks stays ceil(numel / C) whatever the addresses are (trailing chunks may be empty).
+static void fill_chunk_records(rg_plan* p, ChunkRec* out) {
+  p->dst_heads = false;
   for (int i = 0; i < p->n_tensors; ++i) {
     const TensorDesc& t = p->host_tensors[(size_t)i];
     const int ss = elem_size(t.src_dtype), ds = elem_size(t.dst_dtype);
+    const int64_t head = tensor_head(t.src, t.dst, ss, ds);
+    if (t.dst != nullptr && t.numel > 0 && head != 0) p->dst_heads = true;
     for (int64_t c = p->chunk_begin[(size_t)i]; c < p->chunk_begin[(size_t)i + 1]; ++c) {
-      const int64_t start = (c - p->chunk_begin[(size_t)i]) * p->chunk_elems;
-      const int64_t rest = t.numel - start;
+      const int64_t j = c - p->chunk_begin[(size_t)i];
+      const int64_t start = j == 0 ? 0 : std::min(t.numel, head + j * p->chunk_elems);
+      const int64_t end = std::min(t.numel, head + (j + 1) * p->chunk_elems);
       ChunkRec& r = out[c];
       r.src = t.src ? static_cast<const char*>(t.src) + start * ss : nullptr;
       r.dst = t.dst ? static_cast<char*>(t.dst) + start * ds : nullptr;
-      r.len = (int32_t)(rest < p->chunk_elems ? rest : p->chunk_elems);
+      r.len = (int32_t)(end - start);
       r.tensor = i;
       r.src_dtype = (int16_t)t.src_dtype;
       r.dst_dtype = (int16_t)t.dst_dtype;
@@ -248,6 +266,8 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->streaming = bytes > (int64_t)256 << 20;
   p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total);
   if (const char* env = getenv("RG_WRITE_TILE_ELEMS")) p->write_tile_elems = atoll(env);
+  if (const char* env = getenv("RG_XCD_REDUCE")) p->xcd_reduce = atoi(env);
+  if (const char* env = getenv("RG_XCD_WRITE")) p->xcd_write = atoi(env);
 
   p->chunk_begin.assign((size_t)n + 1, 0);
   for (int i = 0; i < n; ++i)
@@ -399,6 +419,8 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   a.n_chunks = p->n_chunks;
   a.tile_elems = (int32_t)p->chunk_elems;
   a.tiles_per_chunk = 1;
+  a.peel_heads = p->dst_heads ? 1 : 0;
+  a.xcd_run = p->xcd_write;
   a.scale = scale;
   a.write_on_overflow = 0;
   a.zero_fill = 0;
@@ -468,12 +490,14 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   PassArgs a = pass_args(p, inv_scale);
   const bool all = ev != nullptr && p->timing_all;
   if (all) RG_HIP(hipEventRecord(ev[0], s));
+  a.xcd_run = p->xcd_reduce;
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
   if (all) RG_HIP(hipEventRecord(ev[1], s));
   RG_HIP(launch_finalize(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
   if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
+  a.xcd_run = p->xcd_write;
   split_for_write(p, a);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, s));
   if (ev) RG_HIP(hipEventRecord(ev[3], s));
@@ -489,7 +513,9 @@ RG_API int rg_step_begin(rg_plan* p, float inv_scale, void* stream) {
   }
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  RG_HIP(launch_pass(kModeReduce, pass_args(p, inv_scale), p->streaming, s));
+  PassArgs a = pass_args(p, inv_scale);
+  a.xcd_run = p->xcd_reduce;
+  RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
   RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
   p->begun_inv_scale = inv_scale;
   return RG_OK;
@@ -599,6 +625,7 @@ RG_API int rg_grad_norm(rg_plan* p, void* stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, 1.0f);
   a.norm_of_source = 1;
+  a.xcd_run = p->xcd_reduce;
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
   RG_HIP(launch_finalize(finalize_args(p, 0.0f, 1), s));
   return RG_OK;
@@ -644,6 +671,8 @@ RG_API int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t nume
   a.single.dst_dtype = (int16_t)dst_dtype;
   a.single_numel = numel;
   a.single_chunk_elems = chunk;
+  a.single_head = tensor_head(src_dev, dst_dev, ss, ds);
+  a.peel_heads = a.single_head != 0 ? 1 : 0;
   a.n_chunks = n_chunks;
   a.tile_elems = kWriteTileElems;
   a.tiles_per_chunk = (int32_t)tiles;

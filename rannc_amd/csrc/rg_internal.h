@@ -61,7 +61,7 @@ static_assert(sizeof(StepResult) == 32, "result block must stay 32 bytes");
 #define RG_ALIGN_BYTES 128
 #endif
 #ifndef RG_WRITE_ALIGN_BYTES
-#define RG_WRITE_ALIGN_BYTES 2
+#define RG_WRITE_ALIGN_BYTES 128
 #endif
 #ifndef RG_DEFAULT_CHUNK_ELEMS
 #define RG_DEFAULT_CHUNK_ELEMS 16384
@@ -74,13 +74,22 @@ constexpr int kReduceElemsPerThread = RG_REDUCE_ELEMS_PER_THREAD;
 constexpr int kWriteElemsPerThread = RG_WRITE_ELEMS_PER_THREAD;
 constexpr int kWriteThreads = RG_WRITE_THREADS;                  // block size of write-only passes
 constexpr int kWriteTileElems = RG_WRITE_TILE_ELEMS;             // writing passes cut each chunk into tiles of this size
-// Per-chunk peel.  The read-only pass peels its source to 128 bytes (one scalar head per
-// 16K-element chunk).  Passes that write do not peel at all (2 = element alignment): gfx950
-// executes element-aligned 128-bit stores, and measured on MI355X that beats peeling the
-// destination to a line boundary (6.1-6.2 vs 5.3-5.7 TB/s for an odd-offset destination),
-// because the scalar head is a dependent load->store round trip inside a very short tile.
+// Alignment.  Measured on MI355X, a pass whose 128-bit stores are not 64-byte aligned loses
+// 9 % (partial-line writes), one whose loads are not 128-byte aligned 3-6 %.  So the side a
+// pass writes decides: chunk boundaries inside a tensor are placed on 128-byte boundaries of
+// its destination (of its source when there is none), which leaves one unaligned head per
+// tensor - not per chunk - to be peeled with scalar accesses; the loads absorb whatever
+// relative misalignment remains.  Read-only passes peel their source per chunk.
+// RG_WRITE_ALIGN_BYTES <= 4 switches the destination peel off (element-aligned vector stores).
 constexpr unsigned kAlignBytes = RG_ALIGN_BYTES;
 constexpr unsigned kWriteAlignBytes = RG_WRITE_ALIGN_BYTES;
+
+// Elements from `addr` to the next `align`-byte boundary (align: power of two; 0 when
+// alignment handling is off).
+__host__ __device__ inline int head_elems(uintptr_t addr, unsigned align, unsigned elem_bytes) {
+  if (align <= 4) return 0;
+  return (int)(((align - (unsigned)(addr & (align - 1))) & (align - 1)) / elem_bytes);
+}
 constexpr int64_t kChunkQuantum = 2048;    // chunk sizes are multiples of this many elements
 constexpr int64_t kMaxChunkElems = 1 << 20;
 constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan
@@ -93,6 +102,9 @@ struct PassArgs {
   ChunkRec single;               // whole-tensor pointers and types (len unused)
   int64_t single_numel;
   int64_t single_chunk_elems;
+  int64_t single_head;           // elements before the first aligned chunk boundary
+  int32_t xcd_run;               // block -> XCD mapping, see pass_kernel
+  int32_t peel_heads;            // writing passes: some destination starts off a boundary
   double* chunk_sumsq;           // [n_chunks * tiles_per_chunk] written when reducing
   int32_t* chunk_bad;            // [n_chunks * tiles_per_chunk] written when reducing
   const StepResult* result;      // non-null: take coef / overflow gate from the device

@@ -254,3 +254,52 @@ def test_accumulate_and_unscale_accumulate(src_name, dst_name):
     with pytest.raises(ValueError, match="itself"):
         TensorPlan([dsts[5]], [dsts[5]]).accumulate(1.0)
     plan.close()
+
+
+@pytest.mark.parametrize("dst_name", ["f32", "bf16"])
+def test_chunk_boundaries_follow_the_destination_alignment(dst_name):
+    """Chunk boundaries inside a tensor sit on 128-byte boundaries of its destination, so the
+    first chunk may be longer than the others and the last one empty; the number of chunks
+    must not depend on the addresses (pointer updates keep the table's size)."""
+    ddt = TORCH_DTYPE[dst_name]
+    chunk = 2048
+    per_line = 128 // torch.empty(0, dtype=ddt).element_size()
+    g = torch.Generator().manual_seed(21)
+    # sizes around multiples of the chunk: a tensor that fits in the lengthened first chunk,
+    # one that needs exactly one more element, and a long one
+    sizes = [chunk, chunk + 1, chunk + per_line - 1, chunk + per_line, 2 * chunk + 3, 10 * chunk + per_line // 2, 7]
+    cpu = [(torch.randn(n, generator=g) * 8).to(torch.float16) for n in sizes]
+    total = sum(sizes) + 4 * per_line
+    src_arena = torch.zeros(total + 64, dtype=torch.float16, device=DEV)
+    plan = None
+    for dst_off in (0, 1, per_line // 2 + 1, per_line - 1):
+        dst_arena = torch.full((total,), 7.0, dtype=ddt, device=DEV)
+        srcs, dsts, o = [], [], dst_off
+        for t in cpu:
+            s = src_arena[o + 3:o + 3 + t.numel()]
+            s.copy_(t)
+            srcs.append(s)
+            dsts.append(dst_arena[o:o + t.numel()])
+            o += t.numel()                                    # no padding: only the first tensor's offset is chosen
+        if plan is None:
+            plan = TensorPlan(srcs, dsts, chunk_elems=chunk)
+            n_chunks = plan.plan.num_chunks
+        else:
+            plan.update(srcs=srcs, dsts=dsts)
+            assert plan.plan.num_chunks == n_chunks
+        plan.fused_step(0.125, math.inf)
+        res = plan.result()
+        want, _ = oracle.unscale_and_check(cpu, 0.125, ddt)
+        assert math.isclose(res.norm, oracle.grad_global_l2_norm(want), rel_tol=1e-6) and res.clipped == 0
+        for d, w in zip(dsts, want):
+            assert_bits_equal(d.cpu(), w, f"offset {dst_off}")
+        out = dst_arena.cpu()
+        assert bool((out[:dst_off] == 7.0).all()) and bool((out[o:] == 7.0).all())      # nothing outside was touched
+        plan.unscale_pack(0.5)
+        want2, _ = oracle.unscale_and_check(cpu, 0.5, ddt)
+        for d, w in zip(dsts, want2):
+            assert_bits_equal(d.cpu(), w, f"unscale_pack offset {dst_off}")
+        plan.zero()
+        out = dst_arena.cpu()
+        assert bool((out[dst_off:o] == 0).all()) and bool((out[:dst_off] == 7.0).all()) and bool((out[o:] == 7.0).all())
+    plan.close()
