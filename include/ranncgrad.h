@@ -191,6 +191,69 @@ int rg_tensor_norms_device_ptr(const rg_plan* plan, const float** out_dev);
 int rg_read_result(rg_plan* plan, rg_step_result* out_host, void* stream);
 int rg_read_tensor_norms(rg_plan* plan, float* out_host, void* stream);
 
+/* ---------------------------------------------------------------- optimizer step */
+
+/* Multi-tensor optimizer step on fp32 parameters, the step that follows the clip: the
+ * reference leaves it to torch.optim (Adam at test/common.py:142,165, SGD at
+ * examples/tutorial.py:28) on the parameters pyrannc/opt.py:205-312 hands it, and under amp
+ * Apex then copies every fp32 master back into its fp16 model parameter
+ * (pyrannc/amp/__init__.py:10-18 keeps the pairing).  One launch updates every tensor of
+ * the table and, where `model_copy[i]` is given, writes round(param) there in the copy's
+ * dtype - the master -> model copy-back without a second pass.
+ *
+ * Table: param, state1, state2 are fp32 and updated in place; grad has dtype grad_dtype[i]
+ * (RG_F32 for master gradients); model_copy[i] may be NULL.  All tensors of a table share
+ * the hyper-parameters and the step count of a call; a parameter without a gradient is
+ * left out of the table (torch.optim skips it).  Adam: state1 = exp_avg, state2 =
+ * exp_avg_sq.  SGD: state1 = momentum buffer (NULL array when momentum == 0), state2 unused. */
+typedef struct rg_optim rg_optim;
+int rg_optim_create(rg_optim** out, int device, int n_tensors, void* const* param, const void* const* grad,
+                    void* const* state1, void* const* state2, void* const* model_copy, const int64_t* numel,
+                    const int* grad_dtype, const int* copy_dtype);
+/* New addresses, same sizes and dtypes; a NULL array keeps the current pointers. */
+int rg_optim_update_pointers(rg_optim* opt, void* const* param, const void* const* grad, void* const* state1,
+                             void* const* state2, void* const* model_copy, void* stream);
+int rg_optim_destroy(rg_optim* opt);
+
+/* Arithmetic of torch.optim.Adam / AdamW (single-tensor form, amsgrad off), in fp32 with
+ * the scalar factors computed in double and rounded once, as ATen does with Python scalars:
+ *   g  = grad * grad_scale            (and * gate->coef; the whole step is skipped when gate->skipped)
+ *   g  = -g                           if maximize
+ *   p  = p * (1 - lr * wd)            if decoupled_weight_decay (AdamW), else g = g + wd * p
+ *   m  = m + (1 - beta1) * (g - m)
+ *   v  = v * beta2 + (1 - beta2) * g * g
+ *   p  = p + (-lr / (1 - beta1^step)) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps)
+ * `step` counts from 1.  `gate` (optional, device pointer from rg_result_device_ptr) lets the
+ * clip coefficient and the overflow skip of a preceding rg_unscale_pack / rg_step_begin be
+ * consumed on the device.  Results agree with torch.optim to rounding (ATen's own CPU and GPU
+ * kernels differ from each other in the last bit); the model copy is bit-exact round-to-
+ * nearest-even of the updated fp32 parameter. */
+typedef struct rg_adam_args {
+  double lr, beta1, beta2, eps, weight_decay;
+  int64_t step;
+  int32_t decoupled_weight_decay;
+  int32_t maximize;
+  float grad_scale;
+  const rg_step_result* gate;
+} rg_adam_args;
+int rg_adam_step(rg_optim* opt, const rg_adam_args* args, void* stream);
+
+/* Arithmetic of torch.optim.SGD:
+ *   g = grad * grad_scale; g = -g if maximize; g = g + wd * p if wd != 0
+ *   momentum != 0:  buf = g on the first step of a buffer (first_step), else
+ *                   buf = momentum * buf + (1 - dampening) * g;
+ *                   g = g + momentum * buf if nesterov, else g = buf
+ *   p = p - lr * g */
+typedef struct rg_sgd_args {
+  double lr, momentum, dampening, weight_decay;
+  int32_t nesterov;
+  int32_t maximize;
+  int32_t first_step;
+  float grad_scale;
+  const rg_step_result* gate;
+} rg_sgd_args;
+int rg_sgd_step(rg_optim* opt, const rg_sgd_args* args, void* stream);
+
 /* ---------------------------------------------------------------- per-kernel timing */
 
 /* Optional profiling aid (no counterpart in the reference, which times with its own

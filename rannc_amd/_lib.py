@@ -25,6 +25,18 @@ class StepResult(C.Structure):
                 ("clipped", C.c_int32), ("skipped", C.c_int32)]
 
 
+class AdamArgs(C.Structure):
+    _fields_ = [("lr", C.c_double), ("beta1", C.c_double), ("beta2", C.c_double), ("eps", C.c_double),
+                ("weight_decay", C.c_double), ("step", C.c_int64), ("decoupled_weight_decay", C.c_int32),
+                ("maximize", C.c_int32), ("grad_scale", C.c_float), ("gate", C.c_void_p)]
+
+
+class SgdArgs(C.Structure):
+    _fields_ = [("lr", C.c_double), ("momentum", C.c_double), ("dampening", C.c_double), ("weight_decay", C.c_double),
+                ("nesterov", C.c_int32), ("maximize", C.c_int32), ("first_step", C.c_int32),
+                ("grad_scale", C.c_float), ("gate", C.c_void_p)]
+
+
 # name -> (restype, argtypes); the complete export list of include/ranncgrad.h
 _vp, _i, _i64, _f = C.c_void_p, C.c_int, C.c_int64, C.c_float
 _pi64, _pi, _pvp = C.POINTER(C.c_int64), C.POINTER(C.c_int), C.POINTER(C.c_void_p)
@@ -58,6 +70,11 @@ SIGNATURES = {
     "rg_tensor_norms_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
     "rg_read_result": (_i, [_vp, C.POINTER(StepResult), _vp]),
     "rg_read_tensor_norms": (_i, [_vp, C.POINTER(C.c_float), _vp]),
+    "rg_optim_create": (_i, [C.POINTER(_vp), _i, _i, _pvp, _pvp, _pvp, _pvp, _pvp, _pi64, _pi, _pi]),
+    "rg_optim_update_pointers": (_i, [_vp, _pvp, _pvp, _pvp, _pvp, _pvp, _vp]),
+    "rg_optim_destroy": (_i, [_vp]),
+    "rg_adam_step": (_i, [_vp, C.POINTER(AdamArgs), _vp]),
+    "rg_sgd_step": (_i, [_vp, C.POINTER(SgdArgs), _vp]),
     "rg_plan_enable_timing": (_i, [_vp, _i]),
     "rg_plan_read_timing": (_i, [_vp, _i, C.POINTER(C.c_float)]),
 }
@@ -245,3 +262,60 @@ def scale_cast_single(src_ptr: Optional[int], dst_ptr: int, numel: int, src_dtyp
 
 def fill_zero(ptr: int, nbytes: int, device: int, stream: int = 0) -> None:
     check(lib.rg_fill_zero(_vp(ptr), nbytes, device, _vp(stream)))
+
+
+# ------------------------------------------------------------------------- optimizer tables
+
+def _ptr_array(ptrs: Optional[Sequence[Optional[int]]], n: int):
+    if ptrs is None:
+        return None
+    if len(ptrs) != n:
+        raise ValueError("pointer arrays differ in length")
+    return (C.c_void_p * max(n, 1))(*[p if p else None for p in ptrs])
+
+
+class OptimTable:
+    """Owner of one ``rg_optim``: parameter / gradient / state / model-copy pointers of the
+    tensors one optimizer launch updates."""
+
+    def __init__(self, device: int, params: Sequence[int], grads: Sequence[int], state1: Optional[Sequence[int]],
+                 state2: Optional[Sequence[int]], copies: Optional[Sequence[Optional[int]]], numels: Sequence[int],
+                 grad_dtypes: Sequence[int], copy_dtypes: Optional[Sequence[int]] = None):
+        n = len(numels)
+        self._handle = _vp()
+        self.n = n
+        self.device = device
+        a_cd = (C.c_int * max(n, 1))(*(copy_dtypes if copy_dtypes is not None else [RG_F32] * n))
+        check(lib.rg_optim_create(C.byref(self._handle), device, n, _ptr_array(params, n), _ptr_array(grads, n),
+                                  _ptr_array(state1, n), _ptr_array(state2, n), _ptr_array(copies, n),
+                                  (C.c_int64 * max(n, 1))(*numels), (C.c_int * max(n, 1))(*grad_dtypes), a_cd))
+
+    def update_pointers(self, params=None, grads=None, state1=None, state2=None, copies=None, stream: int = 0) -> None:
+        n = self.n
+        check(lib.rg_optim_update_pointers(self._handle, _ptr_array(params, n), _ptr_array(grads, n),
+                                           _ptr_array(state1, n), _ptr_array(state2, n), _ptr_array(copies, n),
+                                           _vp(stream)))
+
+    def adam_step(self, lr: float, beta1: float, beta2: float, eps: float, weight_decay: float, step: int,
+                  decoupled: bool = False, maximize: bool = False, grad_scale: float = 1.0, gate: int = 0,
+                  stream: int = 0) -> None:
+        a = AdamArgs(lr, beta1, beta2, eps, weight_decay, step, int(decoupled), int(maximize), grad_scale, gate or None)
+        check(lib.rg_adam_step(self._handle, C.byref(a), _vp(stream)))
+
+    def sgd_step(self, lr: float, momentum: float = 0.0, dampening: float = 0.0, weight_decay: float = 0.0,
+                 nesterov: bool = False, maximize: bool = False, first_step: bool = False, grad_scale: float = 1.0,
+                 gate: int = 0, stream: int = 0) -> None:
+        a = SgdArgs(lr, momentum, dampening, weight_decay, int(nesterov), int(maximize), int(first_step), grad_scale,
+                    gate or None)
+        check(lib.rg_sgd_step(self._handle, C.byref(a), _vp(stream)))
+
+    def close(self) -> None:
+        if self._handle:
+            lib.rg_optim_destroy(self._handle)
+            self._handle = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -186,6 +186,10 @@ def _lazy_init_maybe_master_weights(optimizer: torch.optim.Optimizer) -> None:
                 stash.all_fp32_from_fp32_params.append(p)
                 new_params.append(p)
         group["params"] = new_params
+    if getattr(optimizer, "writes_model_copies", False) and stash.all_fp16_params:
+        # a fused optimizer writes model = half(master) from its step kernel
+        optimizer.set_model_copies(stash.all_fp32_from_fp16_params, [p.detach() for p in stash.all_fp16_params])
+        stash.optimizer_copies_back = True
 
 
 def master_params(optimizer: torch.optim.Optimizer) -> Iterator[torch.Tensor]:
@@ -231,7 +235,8 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
             return None
         finish_unscale(optimizer)
         ret = old_step(*args, **kwargs)
-        _master_to_model(optimizer)
+        if not getattr(stash, "optimizer_copies_back", False):
+            _master_to_model(optimizer)
         stash.norm_is_fresh = False
         return ret
 

@@ -9,6 +9,7 @@
 #include <new>
 #include <vector>
 
+#include "rg_host.h"
 #include "rg_internal.h"
 
 namespace rg {
@@ -21,43 +22,6 @@ void set_error(const char* fmt, ...) {
   vsnprintf(g_error, sizeof(g_error), fmt, ap);
   va_end(ap);
 }
-
-static int hip_fail(hipError_t e, const char* what) {
-  set_error("%s: %s", what, hipGetErrorString(e));
-  return RG_EHIP;
-}
-
-#define RG_HIP(call)                                  \
-  do {                                                \
-    hipError_t e_ = (call);                           \
-    if (e_ != hipSuccess) return hip_fail(e_, #call); \
-  } while (0)
-
-static inline int elem_size(int dtype) {
-  switch (dtype) {
-    case RG_F32: return 4;
-    case RG_F16: return 2;
-    case RG_BF16: return 2;
-    default: return -1;
-  }
-}
-
-static inline int64_t round_up(int64_t x, int64_t q) { return (x + q - 1) / q * q; }
-
-// Makes the plan's device current for the scope of a call and restores the caller's.
-class DeviceGuard {
- public:
-  explicit DeviceGuard(int device) : prev_(-1), changed_(false) {
-    if (hipGetDevice(&prev_) == hipSuccess && prev_ != device) changed_ = (hipSetDevice(device) == hipSuccess);
-  }
-  ~DeviceGuard() {
-    if (changed_) (void)hipSetDevice(prev_);
-  }
-
- private:
-  int prev_;
-  bool changed_;
-};
 
 }  // namespace rg
 
@@ -109,14 +73,6 @@ struct rg_plan {
   int64_t timing_count = 0;
   bool timing_all = true;  // false: only the write pass is bracketed (two records per step)
 };
-
-static int check_pointer(const void* p, int esz, const char* which, int i) {
-  if (p != nullptr && (reinterpret_cast<uintptr_t>(p) % (uintptr_t)esz) != 0) {
-    set_error("%s[%d] = %p is not aligned to its %d-byte element", which, i, p, esz);
-    return RG_EALIGN;
-  }
-  return RG_OK;
-}
 
 // Elements of a tensor before the first 128-byte boundary of the side its passes write
 // (the destination; the source of a plan without destinations).

@@ -1,0 +1,167 @@
+"""Optimizers whose step is one launch of the HIP library over all parameters, with the
+fp32 master -> fp16/bf16 model copy folded in.
+
+The reference leaves the step to ``torch.optim`` (``optim.Adam`` at ``test/common.py:142,165``,
+``optim.SGD`` at ``examples/tutorial.py:28``), patched by ``pyrannc/opt.py:205-312``; under amp
+Apex then copies every master into its model parameter.  ``FusedAdam`` / ``FusedAdamW`` /
+``FusedSGD`` keep ``torch.optim.Adam`` / ``AdamW`` / ``SGD``'s constructor arguments, parameter
+groups and state layout (``step``, ``exp_avg``, ``exp_avg_sq``; ``momentum_buffer``), so state
+dicts, ``patch_optimizer`` and the checkpoint slicing of ``pyrannc/opt.py:186-202`` work on
+them unchanged.  There is no CPU path: parameters must live on the GPU.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from . import _lib
+from .multi_tensor import dtype_code, stream_handle
+
+
+class _FusedBase(torch.optim.Optimizer):
+    def __init__(self, params, defaults):
+        super().__init__(params, defaults)
+        self._tables: Dict[Tuple, Tuple[_lib.OptimTable, Tuple, List]] = {}
+        self._model_copies: Dict[int, torch.Tensor] = {}
+        #: device pointer of an ``rg_step_result`` (``TensorPlan.plan.result_device_ptr()``): the step
+        #: multiplies the gradients by its clip coefficient and does nothing when it says "skipped"
+        self.gate: int = 0
+        #: every gradient is multiplied by this first
+        self.grad_scale: float = 1.0
+
+    # -- model copies (amp): written by the step kernel instead of a separate copy pass
+    writes_model_copies = True
+
+    def set_model_copies(self, masters, models) -> None:
+        """``models[i]`` (fp16/bf16/fp32, same size) receives ``round(masters[i])`` at every step."""
+        for m, c in zip(masters, models):
+            if c.numel() != m.numel() or not c.is_contiguous() or c.device != m.device:
+                raise ValueError("model copy must be a contiguous tensor of the master's size and device")
+            dtype_code(c.dtype)
+            self._model_copies[id(m)] = c
+        self._tables.clear()
+
+    def _check_param(self, p: torch.Tensor) -> None:
+        if p.dtype != torch.float32:
+            raise ValueError(f"fused optimizers step fp32 parameters (masters), got {p.dtype}")
+        if not p.is_cuda or not p.is_contiguous():
+            raise ValueError("fused optimizers need contiguous GPU parameters")
+        if p.grad.is_sparse:
+            raise ValueError("sparse gradients are not supported")
+        if not p.grad.is_contiguous() or p.grad.device != p.device or p.grad.numel() != p.numel():
+            raise ValueError("gradient must be contiguous, on the parameter's device and of its size")
+
+    def _table(self, key: Tuple, params: List[torch.Tensor], state1: Optional[List[torch.Tensor]],
+               state2: Optional[List[torch.Tensor]]) -> _lib.OptimTable:
+        """Table for this exact list of parameters, re-pointed when any address moved."""
+        copies = [self._model_copies.get(id(p)) for p in params]
+        ptrs = (tuple(p.data_ptr() for p in params), tuple(p.grad.data_ptr() for p in params),
+                tuple(s.data_ptr() for s in state1) if state1 is not None else None,
+                tuple(s.data_ptr() for s in state2) if state2 is not None else None,
+                tuple(c.data_ptr() if c is not None else 0 for c in copies))
+        hit = self._tables.get(key)
+        dev = params[0].device
+        if hit is None:
+            table = _lib.OptimTable(dev.index, ptrs[0], ptrs[1], ptrs[2], ptrs[3],
+                                    ptrs[4] if any(ptrs[4]) else None, [p.numel() for p in params],
+                                    [dtype_code(p.grad.dtype) for p in params],
+                                    [dtype_code(c.dtype) if c is not None else _lib.RG_F32 for c in copies])
+        else:
+            table, old, _ = hit
+            if old != ptrs:
+                table.update_pointers(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[4] if any(ptrs[4]) else None,
+                                      stream_handle(dev))
+        # the table borrows raw pointers: keep what it points at alive
+        self._tables[key] = (table, ptrs, [params, [p.grad for p in params], state1, state2, copies])
+        return table
+
+
+class FusedAdam(_FusedBase):
+    """``torch.optim.Adam`` (amsgrad off) as one launch per parameter group."""
+
+    _decoupled = False
+
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, maximize=False):
+        if lr < 0 or eps < 0 or not 0 <= betas[0] < 1 or not 0 <= betas[1] < 1 or weight_decay < 0:
+            raise ValueError("invalid Adam hyper-parameters")
+        super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, maximize=maximize))
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for gi, group in enumerate(self.param_groups):
+            by_step: Dict[int, List[torch.Tensor]] = {}
+            for p in group["params"]:
+                if p.grad is None:
+                    continue
+                self._check_param(p)
+                st = self.state[p]
+                if len(st) == 0:
+                    st["step"] = torch.tensor(0.0, dtype=torch.float32)
+                    st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                    st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                st["step"] += 1
+                by_step.setdefault(int(st["step"]), []).append(p)
+            for step, ps in by_step.items():
+                ms = [self.state[p]["exp_avg"] for p in ps]
+                vs = [self.state[p]["exp_avg_sq"] for p in ps]
+                table = self._table((gi, tuple(id(p) for p in ps)), ps, ms, vs)
+                b1, b2 = group["betas"]
+                table.adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], step,
+                                decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
+                                gate=self.gate, stream=stream_handle(ps[0].device))
+        return loss
+
+
+class FusedAdamW(FusedAdam):
+    """``torch.optim.AdamW``: weight decay applied to the parameter, not the gradient."""
+
+    _decoupled = True
+
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, maximize=False):
+        super().__init__(params, lr, betas, eps, weight_decay, maximize)
+
+
+class FusedSGD(_FusedBase):
+    """``torch.optim.SGD`` as one launch per parameter group (two on the step that creates
+    momentum buffers for only some of the parameters)."""
+
+    def __init__(self, params, lr=1e-3, momentum=0.0, dampening=0.0, weight_decay=0.0, nesterov=False, maximize=False):
+        if lr < 0 or momentum < 0 or weight_decay < 0:
+            raise ValueError("invalid SGD hyper-parameters")
+        if nesterov and (momentum <= 0 or dampening != 0):
+            raise ValueError("Nesterov momentum requires a momentum and zero dampening")
+        super().__init__(params, dict(lr=lr, momentum=momentum, dampening=dampening, weight_decay=weight_decay,
+                                      nesterov=nesterov, maximize=maximize))
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for gi, group in enumerate(self.param_groups):
+            fresh, seasoned = [], []
+            for p in group["params"]:
+                if p.grad is None:
+                    continue
+                self._check_param(p)
+                st = self.state[p]
+                if group["momentum"] != 0 and st.get("momentum_buffer") is None:
+                    st["momentum_buffer"] = torch.empty_like(p, memory_format=torch.preserve_format)
+                    fresh.append(p)
+                else:
+                    seasoned.append(p)
+            for first, ps in ((True, fresh), (False, seasoned)):
+                if not ps:
+                    continue
+                bufs = [self.state[p]["momentum_buffer"] for p in ps] if group["momentum"] != 0 else None
+                table = self._table((gi, first, tuple(id(p) for p in ps)), ps, bufs, None)
+                table.sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
+                               group["nesterov"], group["maximize"], first_step=first, grad_scale=self.grad_scale,
+                               gate=self.gate, stream=stream_handle(ps[0].device))
+        return loss
