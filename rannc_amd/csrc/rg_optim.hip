@@ -54,9 +54,19 @@ struct OptArgs {
   OptConst c;
 };
 
-constexpr int kOptThreads = 128;
-constexpr int kOptTileElems = 1024;
+#ifndef RG_OPT_THREADS
+#define RG_OPT_THREADS 128
+#endif
+#ifndef RG_OPT_TILE_ELEMS
+#define RG_OPT_TILE_ELEMS 1024
+#endif
+#ifndef RG_OPT_UNROLL
+#define RG_OPT_UNROLL 1
+#endif
+constexpr int kOptThreads = RG_OPT_THREADS;
+constexpr int kOptTileElems = RG_OPT_TILE_ELEMS;
 constexpr int kOptE = 4;    // elements per lane per instruction
+constexpr int kOptU = RG_OPT_UNROLL;   // vectors per array a lane has in flight
 
 template <int ALGO>
 __device__ __forceinline__ void update_one(float& p, float g, float& s1, float& s2, const OptConst& c, float gscale) {
@@ -69,8 +79,13 @@ __device__ __forceinline__ void update_one(float& p, float g, float& s1, float& 
     s1 = __builtin_fmaf(c.lerp_coeff, g - s1, c.lerp_from_end ? g : s1);
     // exp_avg_sq.mul_(beta2).addcmul_(g, g, value = 1 - beta2)
     s2 = __builtin_fmaf(c.one_minus_beta2 * g, g, s2 * c.beta2);
+#ifdef RG_ADAM_FAST_MATH   // diagnostic build only: approximate sqrt / reciprocal
+    const float denom = __builtin_amdgcn_sqrtf(s2) * c.bias2_sqrt + c.eps;
+    p = p + (c.neg_step_size * s1) * __builtin_amdgcn_rcpf(denom);
+#else
     const float denom = sqrtf(s2) / c.bias2_sqrt + c.eps;
     p = p + (c.neg_step_size * s1) / denom;
+#endif
   } else {
     if (c.weight_decay != 0.0f) g = __builtin_fmaf(c.weight_decay, p, g);
     if (c.has_momentum) {
@@ -105,7 +120,7 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
   char* s1p = r.state1 ? reinterpret_cast<char*>(r.state1) + (size_t)start * 4 : nullptr;
   char* s2p = r.state2 ? reinterpret_cast<char*>(r.state2) + (size_t)start * 4 : nullptr;
   char* cp = kCopy ? reinterpret_cast<char*>(r.copy) + (size_t)start * CS : nullptr;
-  const bool use_s1 = ALGO == kAdam || s1p != nullptr;
+  const bool use_s1 = ALGO == kAdam || (c.has_momentum != 0 && s1p != nullptr);
   const int tid = threadIdx.x;
 
   // Unaligned head of the parameter (at most one per tensor: chunk and tile boundaries sit
@@ -128,12 +143,15 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
     if (kCopy) store1<CD>(cp + (size_t)i * CS, p);
   }
 
-  for (int e = head + tid * E; e < tail0; e += T * E) {
-    const Raw<RG_F32, E> rp = Mem<RG_F32, E, NT>::load(pp + (size_t)e * 4);
-    const Raw<G, E> rg = Mem<G, E, NT>::load(gp + (size_t)e * GS);
-    Raw<RG_F32, E> r1 = rp, r2 = rp;
+  auto vec = [&](int e, Raw<RG_F32, E>& rp, Raw<G, E>& rg, Raw<RG_F32, E>& r1, Raw<RG_F32, E>& r2) {
+    rp = Mem<RG_F32, E, NT>::load(pp + (size_t)e * 4);
+    rg = Mem<G, E, NT>::load(gp + (size_t)e * GS);
+    r1 = rp;
+    r2 = rp;
     if (use_s1) r1 = Mem<RG_F32, E, NT>::load(s1p + (size_t)e * 4);
     if (ALGO == kAdam) r2 = Mem<RG_F32, E, NT>::load(s2p + (size_t)e * 4);
+  };
+  auto finish = [&](int e, const Raw<RG_F32, E>& rp, const Raw<G, E>& rg, const Raw<RG_F32, E>& r1, const Raw<RG_F32, E>& r2) {
     float p[E], g[E], s1[E], s2[E];
     Codec<RG_F32, E>::unpack(rp, p);
     Codec<G, E>::unpack(rg, g);
@@ -145,6 +163,23 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
     if (use_s1) Mem<RG_F32, E, NT>::store(s1p + (size_t)e * 4, Codec<RG_F32, E>::pack(s1));
     if (ALGO == kAdam) Mem<RG_F32, E, NT>::store(s2p + (size_t)e * 4, Codec<RG_F32, E>::pack(s2));
     if constexpr (kCopy) Mem<CD, E, NT>::store(cp + (size_t)e * CS, Codec<CD, E>::pack(p));
+  };
+  constexpr int U = kOptU;
+  constexpr int kIter = T * E * U;
+  int base = head;
+  for (; base + kIter <= tail0; base += kIter) {     // all loads of U steps in flight together
+    Raw<RG_F32, E> rp[U], r1[U], r2[U];
+    Raw<G, E> rg[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) vec(base + (u * T + tid) * E, rp[u], rg[u], r1[u], r2[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) finish(base + (u * T + tid) * E, rp[u], rg[u], r1[u], r2[u]);
+  }
+  for (int e = base + tid * E; e < tail0; e += T * E) {
+    Raw<RG_F32, E> rp, r1, r2;
+    Raw<G, E> rg;
+    vec(e, rp, rg, r1, r2);
+    finish(e, rp, rg, r1, r2);
   }
 }
 
