@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # HBM traffic per launch of the dominant kernel (the write pass), from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs of this same command, each scaled by what the counter reads for
 # a plain 1 GiB copy (profiles/fused_step_c2_bert_large_hbm_traffic.txt).  Missing = not measured.
-MEASURED_TRAFFIC_BYTES = {"c2_bert_large": 2021546116}
+MEASURED_TRAFFIC_BYTES = {"c2_bert_large": 2021550504}
 
 
 def parse_args():
@@ -32,6 +32,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_bert_large")
+    ap.add_argument("--op", default="fused_step", choices=["fused_step", "adam", "sgd"],
+                    help="fused_step (default: the graded metric) or the optimizer step that follows it")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--chunk-elems", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -97,6 +99,115 @@ def cpu_baseline(cfg, seed: int, budget_s: float):
     }
 
 
+def bench_optimizer(args, cfg, torch, dev) -> dict:
+    """Adam (+ bf16/fp16 model copy) or plain SGD over the workload's tensors: fp32 masters, fp32
+    master gradients laid out as views of one packed bucket, separately allocated moments."""
+    from rannc_amd import _lib
+    from rannc_amd.multi_tensor import stream_handle
+    from rannc_amd.workloads import make_grads
+
+    grads, _ = make_grads(cfg, args.seed, device=str(dev))
+    shapes = [g.shape for g in grads]
+    copy_dt = grads[0].dtype if grads[0].dtype != torch.float32 else torch.bfloat16
+    del grads
+    n = sum(torch.Size(sh).numel() for sh in shapes)
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    bucket = torch.randn(n, device=dev, generator=gen) * 1e-2
+    gviews, off = [], 0
+    for sh in shapes:
+        k = torch.Size(sh).numel()
+        gviews.append(bucket.narrow(0, off, k))
+        off += k
+    params = [torch.randn(sh, device=dev, generator=gen) for sh in shapes]
+    adam = args.op == "adam"
+    m = [torch.zeros_like(p) for p in params] if adam else None
+    v = [torch.zeros_like(p) for p in params] if adam else None
+    copies = [torch.zeros(sh, device=dev, dtype=copy_dt) for sh in shapes]
+    code = {torch.float16: _lib.RG_F16, torch.bfloat16: _lib.RG_BF16}[copy_dt]
+    table = _lib.OptimTable(0, [t.data_ptr() for t in params], [t.data_ptr() for t in gviews],
+                            [t.data_ptr() for t in m] if adam else None, [t.data_ptr() for t in v] if adam else None,
+                            [t.data_ptr() for t in copies], [t.numel() for t in params], [_lib.RG_F32] * len(params),
+                            [code] * len(params))
+    st = stream_handle(dev)
+    count = [0]
+
+    def step():
+        count[0] += 1
+        if adam:
+            table.adam_step(1e-3, 0.9, 0.999, 1e-8, 0.0, count[0], stream=st)
+        else:
+            table.sgd_step(0.01, stream=st)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()                       # the kernel is launched on torch's current stream, where these events sit
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    launch_ms = e0.elapsed_time(e1) / args.steps
+    bytes_per_elem = (16 + 12 + 2) if adam else (8 + 4 + 2)
+    step_bytes = bytes_per_elem * n
+    step_s = elapsed / args.steps
+    achieved = step_bytes / (launch_ms * 1e-3) / 1e9
+    out = {
+        "metric": f"achieved HBM GB/s for the multi-tensor {args.op} step with model copy-back",
+        "value": round(step_bytes / step_s / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": cfg.key, "op": args.op, "tensors": len(params), "elements": n,
+                   "bytes_per_elem": bytes_per_elem, "model_copy_dtype": str(copy_dt), "seed": args.seed},
+        "pct_of_hbm_peak": round(100.0 * step_bytes / step_s / 1e9 / HBM_PEAK_GBPS, 2),
+        "roofline": {"bound": "hbm", "kernel": f"optim_kernel<{args.op}, streaming>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": step_bytes, "avg_launch_ms": round(launch_ms, 4)},
+    }
+    table.close()
+    del params, m, v, copies, bucket, gviews
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_optimizer(args.op, shapes, args.seed, args.cpu_seconds, bytes_per_elem)
+    return out
+
+
+def cpu_baseline_optimizer(op: str, shapes, seed: int, budget_s: float, bytes_per_elem: int) -> dict:
+    """torch.optim's op sequence (the oracle restates it; bit-identical to the library) on the
+    host cores, over as many leading tensors of the workload as fit the time budget."""
+    import torch
+    from oracle import optim as oracle_optim
+    torch.set_num_threads(os.cpu_count() or 1)
+    gen = torch.Generator().manual_seed(seed)
+    take, total = [], 0
+    for sh in shapes:
+        take.append(sh)
+        total += torch.Size(sh).numel()
+        if total >= 64_000_000:
+            break
+    p = [torch.randn(sh, generator=gen) for sh in take]
+    g = [torch.randn(sh, generator=gen) * 1e-2 for sh in take]
+    m = [torch.zeros_like(t) for t in p]
+    v = [torch.zeros_like(t) for t in p]
+    best, reps, t_start = float("inf"), 0, time.perf_counter()
+    while reps < 5 and (reps == 0 or time.perf_counter() - t_start < budget_s):
+        t0 = time.perf_counter()
+        if op == "adam":
+            oracle_optim.adam_step(p, g, m, v, reps + 1)
+        else:
+            oracle_optim.sgd_step(p, g, None, 0.01)
+        copies = [oracle_optim.model_copy(t, torch.bfloat16) for t in p]
+        best = min(best, time.perf_counter() - t0)
+        reps += 1
+        del copies
+    return {"value": round(bytes_per_elem * total / best / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "cpu": cpu_model(),
+            "sample": f"first {len(take)} tensors ({total} elements) of the workload, best of {reps} passes of "
+                      f"torch.optim's per-tensor op sequence + master->bf16 copy"}
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -115,6 +226,9 @@ def main() -> int:
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     cfg = step_config(args.workload)
+    if args.op != "fused_step":
+        print(json.dumps(bench_optimizer(args, cfg, torch, dev)), flush=True)
+        return 0
     if args.calibrate_copy:
         a = torch.empty(256 << 20, dtype=torch.float32, device=dev).fill_(1.0)
         b = torch.empty_like(a)
