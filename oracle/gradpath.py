@@ -438,3 +438,29 @@ def unscale_accumulate(master_grads: Sequence[torch.Tensor], model_grads: Sequen
             overflow = 1
         m.copy_((m.to(torch.float32) + gf * scale).to(m.dtype))
     return overflow
+
+
+# --------------------------------------------------------------------------- shared parameters
+
+def sum_clone_grads(param_grads: List[Optional[torch.Tensor]],
+                    clone_grads: Sequence[Sequence[Optional[torch.Tensor]]]) -> None:
+    """``TorchDriver::backward``, "backward_sum_paramgrad" (``src/torch/TorchDriver.cpp:781-822``):
+    per shared parameter ``grad_sum = zeros; for each clone with a gradient: grad_sum.add_(g);
+    g.zero_()`` in clone order, then ``grad.add_(grad_sum)`` or, when the parameter has no
+    gradient yet, ``grad = copy of grad_sum``.  In place on the lists given.  Additions happen
+    in the tensors' own dtype (ATen computes a 16-bit ``add_`` in fp32 and rounds once)."""
+    for i, clones in enumerate(clone_grads):
+        if not clones:
+            continue
+        ref = next((g for g in clones if g is not None), param_grads[i])
+        if ref is None:
+            continue
+        grad_sum = torch.zeros_like(ref)
+        for g in clones:
+            if g is not None:
+                grad_sum.add_(g)
+                g.zero_()
+        if param_grads[i] is not None:
+            param_grads[i].add_(grad_sum)
+        else:
+            param_grads[i] = grad_sum.clone()

@@ -354,3 +354,39 @@ def test_patch_optimizer_zero_mode_bookkeeping():
     assert sorted(sd.keys()) == ["param_groups", "state"]
     with pytest.raises(ValueError, match="enable_apex_amp"):
         rannc_amd.RaNNCModule(model, opt, enable_zero=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_clone_grad_summer_matches_the_reference_loop(dtype):
+    from rannc_amd.shared_params import CloneGradSummer
+    g = torch.Generator().manual_seed(31)
+    shapes = [(1000,), (33, 7), (70001,), (5,)]
+    n_clones = [2, 3, 0, 1]
+    params = [torch.zeros(s, dtype=dtype, device=DEV, requires_grad=True) for s in shapes]
+    clones = [[torch.zeros(s, dtype=dtype, device=DEV, requires_grad=True) for _ in range(k)] for s, k in zip(shapes, n_clones)]
+    summer = CloneGradSummer(params, clones)
+    for step in range(2):                    # second round: parameter gradients exist and are added to
+        cpu_clone_grads = []
+        for i, cl in enumerate(clones):
+            row = []
+            for k, c in enumerate(cl):
+                if (i, k) == (1, 1) and step == 0:
+                    c.grad = None            # a clone that received no gradient
+                    row.append(None)
+                else:
+                    val = (torch.randn(shapes[i], generator=g) * 300).to(dtype)
+                    c.grad = val.to(DEV)
+                    row.append(val.clone())
+            cpu_clone_grads.append(row)
+        cpu_param_grads = [None if p.grad is None else p.grad.cpu().clone() for p in params]
+        summer.sum_into_params()
+        oracle.sum_clone_grads(cpu_param_grads, cpu_clone_grads)
+        for i, p in enumerate(params):
+            if n_clones[i] == 0:
+                assert p.grad is None
+                continue
+            assert_bits_equal(p.grad.cpu(), cpu_param_grads[i], f"param {i} step {step}")
+            for c in clones[i]:
+                assert c.grad is None or bool((c.grad == 0).all())
+    with pytest.raises(ValueError):
+        CloneGradSummer([params[0]], [[params[1]]])

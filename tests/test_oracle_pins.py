@@ -317,3 +317,19 @@ def test_unscale_accumulate_is_two_roundings():
     assert torch.equal(z, model.float())
     model[5] = float("nan")
     assert oracle.unscale_accumulate([master.clone()], [model], 0.5) == 1
+
+
+def test_sum_clone_grads_order_and_rounding():
+    # fp16: (a + b) + c is rounded after every addition, in clone order
+    a = torch.tensor([2048.0, 1.0], dtype=torch.float16)
+    b = torch.tensor([1.0, 1.0], dtype=torch.float16)
+    c = torch.tensor([1.0, -2.0], dtype=torch.float16)
+    grads = [None]
+    clones = [[a.clone(), b.clone(), c.clone()]]
+    oracle.sum_clone_grads(grads, clones)
+    # 2048 + 1 = 2049 -> rounds to 2048 (ulp 2), again + 1 -> 2048; a sum in higher precision would give 2050
+    assert grads[0].tolist() == [2048.0, 0.0]
+    assert all(float(g.abs().sum()) == 0.0 for g in clones[0])           # clone grads are cleared
+    have = [torch.tensor([10.0, 10.0], dtype=torch.float16)]
+    oracle.sum_clone_grads(have, [[a.clone(), None, c.clone()]])
+    assert have[0].tolist() == [2058.0, 9.0]                              # grad_sum = [2048, -1] is added to the existing gradient
