@@ -38,6 +38,7 @@ struct rg_plan {
   int64_t write_tile_elems = kWriteTileElems;
   int xcd_reduce = 64;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
   int xcd_write = 0;
+  int64_t reduce_tile_factor = 0;    // tile of a reducing + writing pass, in write tiles (0 = per operation)
   float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
   std::vector<TensorDesc> host_tensors;
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
@@ -224,6 +225,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   if (const char* env = getenv("RG_WRITE_TILE_ELEMS")) p->write_tile_elems = atoll(env);
   if (const char* env = getenv("RG_XCD_REDUCE")) p->xcd_reduce = atoi(env);
   if (const char* env = getenv("RG_XCD_WRITE")) p->xcd_write = atoi(env);
+  if (const char* env = getenv("RG_REDUCE_TILE_FACTOR")) p->reduce_tile_factor = atoll(env);
 
   p->chunk_begin.assign((size_t)n + 1, 0);
   for (int i = 0; i < n; ++i)
@@ -250,8 +252,9 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   const size_t max_tiles = (size_t)((p->chunk_elems + p->write_tile_elems - 1) / p->write_tile_elems);
   const size_t o_sumsq = carve(nc * sizeof(double));
   const size_t o_bad = carve(nc * sizeof(int32_t));
-  const size_t o_tile_sumsq = carve(nc * max_tiles * sizeof(double));
-  const size_t o_tile_bad = carve(nc * max_tiles * sizeof(int32_t));
+  const size_t tile_partials = nc * max_tiles;
+  const size_t o_tile_sumsq = carve(tile_partials * sizeof(double));
+  const size_t o_tile_bad = carve(tile_partials * sizeof(int32_t));
   const size_t o_tnorm = carve(nt * sizeof(float));
   const size_t o_tsq = carve(nt * sizeof(double));
   const size_t o_tbad = carve(nt * sizeof(int32_t));
@@ -396,6 +399,7 @@ static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_o
   f.n_tensors = p->n_tensors;
   f.max_norm = max_norm;
   f.ignore_overflow = ignore_overflow;
+  f.partials_per_chunk = 1;
   return f;
 }
 
@@ -407,6 +411,28 @@ static void split_for_write(const rg_plan* p, PassArgs& a) {
     a.tile_elems = (int32_t)tile;
     a.tiles_per_chunk = (int32_t)((p->chunk_elems + tile - 1) / tile);
   }
+}
+
+// One pass that both reduces and writes, over tiles of each chunk: every tile leaves its own
+// partial sum, and the per-tensor finalize adds the tile partials directly.
+static int tiled_reduce_write(rg_plan* p, PassArgs& a, int mode, hipStream_t s) {
+  split_for_write(p, a);
+  // measured on MI355X: twice the write tile is best for unscale+pack, the plain write tile when accumulating
+  const int64_t factor = p->reduce_tile_factor > 0 ? p->reduce_tile_factor : ((mode & kModeAccumulate) ? 1 : 2);
+  if (a.tiles_per_chunk > 1 && factor > 1 && a.tile_elems * factor <= p->chunk_elems) {
+    // every tile of this pass also pays a block-wide reduction: a larger tile amortises it
+    a.tile_elems = (int32_t)(a.tile_elems * factor);
+    a.tiles_per_chunk = (int32_t)((p->chunk_elems + a.tile_elems - 1) / a.tile_elems);
+  }
+  FinalizeArgs f = finalize_args(p, 0.0f, 0);
+  a.chunk_sumsq = p->d_tile_sumsq;
+  a.chunk_bad = p->d_tile_bad;
+  f.chunk_sumsq = p->d_tile_sumsq;
+  f.chunk_bad = p->d_tile_bad;
+  f.partials_per_chunk = a.tiles_per_chunk;
+  RG_HIP(launch_pass(mode, a, p->streaming, s));
+  RG_HIP(launch_finalize(f, s));
+  return RG_OK;
 }
 
 // Which pointers an operation dereferences.
@@ -506,22 +532,7 @@ RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, inv_scale);
-  split_for_write(p, a);
-  if (a.tiles_per_chunk > 1 && a.tile_elems * 2 <= p->chunk_elems) {
-    // every tile of this pass also pays a block-wide reduction: twice the tile amortises it
-    a.tile_elems *= 2;
-    a.tiles_per_chunk = (int32_t)((p->chunk_elems + a.tile_elems - 1) / a.tile_elems);
-  }
-  if (a.tiles_per_chunk > 1) {
-    a.chunk_sumsq = p->d_tile_sumsq;
-    a.chunk_bad = p->d_tile_bad;
-  }
-  RG_HIP(launch_pass(kModeReduce | kModeWrite, a, p->streaming, s));
-  if (a.tiles_per_chunk > 1)
-    RG_HIP(launch_fold_tiles(p->d_tile_sumsq, p->d_tile_bad, p->d_chunk_sumsq, p->d_chunk_bad, p->n_chunks,
-                             a.tiles_per_chunk, s));
-  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
-  return RG_OK;
+  return tiled_reduce_write(p, a, kModeReduce | kModeWrite, s);
 }
 
 static int check_not_in_place(const rg_plan* p, const char* op) {
@@ -557,21 +568,7 @@ RG_API int rg_unscale_accumulate(rg_plan* p, float inv_scale, void* stream) {
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, inv_scale);
-  split_for_write(p, a);
-  if (a.tiles_per_chunk > 1 && a.tile_elems * 2 <= p->chunk_elems) {
-    a.tile_elems *= 2;
-    a.tiles_per_chunk = (int32_t)((p->chunk_elems + a.tile_elems - 1) / a.tile_elems);
-  }
-  if (a.tiles_per_chunk > 1) {
-    a.chunk_sumsq = p->d_tile_sumsq;
-    a.chunk_bad = p->d_tile_bad;
-  }
-  RG_HIP(launch_pass(kModeReduce | kModeWrite | kModeAccumulate, a, p->streaming, s));
-  if (a.tiles_per_chunk > 1)
-    RG_HIP(launch_fold_tiles(p->d_tile_sumsq, p->d_tile_bad, p->d_chunk_sumsq, p->d_chunk_bad, p->n_chunks,
-                             a.tiles_per_chunk, s));
-  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
-  return RG_OK;
+  return tiled_reduce_write(p, a, kModeReduce | kModeWrite | kModeAccumulate, s);
 }
 
 RG_API int rg_grad_norm(rg_plan* p, void* stream) {

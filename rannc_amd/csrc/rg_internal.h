@@ -128,15 +128,13 @@ struct FinalizeArgs {
   int32_t n_tensors;
   float max_norm;
   int32_t ignore_overflow;  // overflow is reported but neither gates the clip nor the write
+  int32_t partials_per_chunk;  // 1, or the tiles per chunk of a tiled reducing pass
 };
 
 // streaming: nontemporal loads/stores (data far larger than the caches).
 hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream);
 hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream);
-// chunk[c] = sum over t of tile[c * tiles_per_chunk + t], in order (after a tiled reducing pass)
-hipError_t launch_fold_tiles(const double* tile_sumsq, const int32_t* tile_bad, double* chunk_sumsq, int32_t* chunk_bad,
-                             int64_t n_chunks, int tiles_per_chunk, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
 
 void set_error(const char* fmt, ...);

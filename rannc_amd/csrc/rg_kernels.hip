@@ -303,47 +303,46 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
   }
 
   if (MODE & kModeReduce) {
-    // Fixed-order combine: 8 lanes of the thread, 64 lanes of the wavefront by shuffle, the
-    // wavefronts through LDS in index order.  Everything past the per-thread fp32 sums is double.
+    // Fixed-order combine: 8 sums of the thread, 64 lanes of the wavefront by DPP row scans.
+    // Everything past the per-thread fp32 sums is double.
+    // A non-finite input makes its square, and so the sum, non-finite; a finite sum therefore
+    // proves every input was finite.  Only when a sum is not finite are the elements looked
+    // at again one by one (the sum can also overflow from finite inputs).
     constexpr int kWaves = T / 64;
     double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
                (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
+    s = wave_total(s);
+    {
+      // One partial per block, the wavefronts combined through LDS in index order.
+      __shared__ double wave_sum[kWaves];
+      if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = s;
+      __syncthreads();
+      double total = wave_sum[0];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off);
-    __shared__ double wave_sum[kWaves];
-    if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = s;
-    __syncthreads();
-    double total = wave_sum[0];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) total += wave_sum[w];
-    // A non-finite input makes its square, and so the chunk's sum, non-finite; a finite sum
-    // therefore proves every input was finite.  Only chunks whose sum is not finite are
-    // looked at again element by element (the sum can also overflow from finite inputs).
-    int bad = 0;
-    if (!(fabs(total) <= 1.79769313486231570e308)) {
-      int mine = 0;
-      if (sp != nullptr) {
-        if (src_kind == RG_F32) mine = rescan_nonfinite<RG_F32, T>(sp, len);
-        else if (src_kind == RG_F16) mine = rescan_nonfinite<RG_F16, T>(sp, len);
-        else mine = rescan_nonfinite<RG_BF16, T>(sp, len);
+      for (int w = 1; w < kWaves; ++w) total += wave_sum[w];
+      int bad = 0;
+      if (!(fabs(total) <= 1.79769313486231570e308)) {
+        int mine = 0;
+        if (sp != nullptr) {
+          if (src_kind == RG_F32) mine = rescan_nonfinite<RG_F32, T>(sp, len);
+          else if (src_kind == RG_F16) mine = rescan_nonfinite<RG_F16, T>(sp, len);
+          else mine = rescan_nonfinite<RG_BF16, T>(sp, len);
+        }
+        bad = __syncthreads_or(mine);
       }
-      bad = __syncthreads_or(mine);
-    }
-    if (threadIdx.x == 0) {
-      a.chunk_sumsq[bid] = total;
-      a.chunk_bad[bid] = bad;
+      if (threadIdx.x == 0) {
+        a.chunk_sumsq[bid] = total;
+        a.chunk_bad[bid] = bad;
+      }
     }
   }
 }
 
-// Fixed-order sum of one value per thread over the block: shuffle tree inside each
+// Fixed-order sum of one value per thread over the block: DPP row scans inside each
 // wavefront, then the wavefront totals through LDS in index order.
 __device__ __forceinline__ void block_sum_or(double& s, int& bad, double* lds_sum, int* lds_bad) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    s += __shfl_down(s, off);
-    bad |= __shfl_down(bad, off);
-  }
+  s = wave_total(s);
+  bad = __any(bad) ? 1 : 0;
   if ((threadIdx.x & 63) == 0) {
     lds_sum[threadIdx.x >> 6] = s;
     lds_bad[threadIdx.x >> 6] = bad;
@@ -362,8 +361,9 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_tensors_kernel(Finaliz
   const int t = blockIdx.x;
   double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
   int bad = 0;
-  const int64_t end = a.tensor_chunk_begin[t + 1];
-  int64_t c = a.tensor_chunk_begin[t] + threadIdx.x;
+  // partials_per_chunk > 1: the pass left one partial per tile, laid out chunk-major
+  const int64_t end = a.tensor_chunk_begin[t + 1] * a.partials_per_chunk;
+  int64_t c = a.tensor_chunk_begin[t] * a.partials_per_chunk + threadIdx.x;
   for (; c + 3 * kBlockThreads < end; c += 4 * kBlockThreads) {
     const double v0 = a.chunk_sumsq[c], v1 = a.chunk_sumsq[c + kBlockThreads];
     const double v2 = a.chunk_sumsq[c + 2 * kBlockThreads], v3 = a.chunk_sumsq[c + 3 * kBlockThreads];
@@ -422,26 +422,6 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_total_kernel(FinalizeA
   }
 }
 
-// After a tiled reducing pass: thread c adds chunk c's tile partials in tile order.
-__global__ __launch_bounds__(kBlockThreads) void fold_tiles_kernel(const double* __restrict__ tile_sumsq,
-                                                                   const int32_t* __restrict__ tile_bad,
-                                                                   double* __restrict__ chunk_sumsq,
-                                                                   int32_t* __restrict__ chunk_bad, int64_t n_chunks,
-                                                                   int tiles_per_chunk) {
-  const int64_t c = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
-  if (c >= n_chunks) return;
-  double s = 0.0;
-  int bad = 0;
-  const double* ts = tile_sumsq + c * tiles_per_chunk;
-  const int32_t* tb = tile_bad + c * tiles_per_chunk;
-  for (int t = 0; t < tiles_per_chunk; ++t) {
-    s += ts[t];
-    bad |= tb[t];
-  }
-  chunk_sumsq[c] = s;
-  chunk_bad[c] = bad;
-}
-
 __global__ __launch_bounds__(kBlockThreads) void fill_zero_kernel(char* p, int64_t nbytes) {
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
   int64_t head = (int64_t)((16u - (unsigned)(a & 15u)) & 15u);
@@ -490,15 +470,6 @@ hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream) {
   if (a.n_tensors > 0)
     hipLaunchKernelGGL(finalize_tensors_kernel, dim3((unsigned)a.n_tensors), dim3(kBlockThreads), 0, stream, a);
   hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
-  return hipGetLastError();
-}
-
-hipError_t launch_fold_tiles(const double* tile_sumsq, const int32_t* tile_bad, double* chunk_sumsq, int32_t* chunk_bad,
-                             int64_t n_chunks, int tiles_per_chunk, hipStream_t stream) {
-  if (n_chunks <= 0) return hipSuccess;
-  const unsigned blocks = (unsigned)((n_chunks + kBlockThreads - 1) / kBlockThreads);
-  hipLaunchKernelGGL(fold_tiles_kernel, dim3(blocks), dim3(kBlockThreads), 0, stream, tile_sumsq, tile_bad, chunk_sumsq,
-                     chunk_bad, n_chunks, tiles_per_chunk);
   return hipGetLastError();
 }
 
