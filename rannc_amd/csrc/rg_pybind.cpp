@@ -167,6 +167,85 @@ class Plan {
   py::object keep_src_, keep_dst_;  // the table points into these tensors
 };
 
+// Table of an optimizer launch: fp32 parameters, their gradients, one or two fp32 state
+// tensors per parameter and (optionally) the low-precision model copies written by the step.
+class Optim {
+ public:
+  Optim(const py::sequence& params, const py::sequence& grads, const py::object& state1, const py::object& state2,
+        const py::object& copies)
+      : keep_(py::make_tuple(params, grads, state1, state2, copies)) {
+    const size_t n = py::len(params);
+    if (py::len(grads) != n) throw std::invalid_argument("params and grads differ in length");
+    std::vector<void*> p, s1, s2, c;
+    std::vector<const void*> g;
+    std::vector<int64_t> numel;
+    std::vector<int> gdt, cdt;
+    auto column = [&](const py::object& o, const char* what, std::vector<void*>& out, std::vector<int>* dtypes, bool need_f32) {
+      if (o.is_none()) return;
+      py::sequence seq = o.cast<py::sequence>();
+      if (py::len(seq) != n) throw std::invalid_argument(std::string(what) + " differs in length from params");
+      for (size_t i = 0; i < n; ++i) {
+        const Ref r = tensor_ref(seq[i], what, i);
+        if (r.defined && (r.numel != numel[i] || r.device != device_))
+          throw std::invalid_argument(std::string(what) + "[" + std::to_string(i) + "] differs in size or device from its parameter");
+        if (r.defined && need_f32 && r.dtype != RG_F32)
+          throw std::invalid_argument(std::string(what) + "[" + std::to_string(i) + "] must be float32");
+        out.push_back(r.ptr);
+        if (dtypes) dtypes->push_back(r.defined ? r.dtype : (int)RG_F32);
+      }
+    };
+    for (size_t i = 0; i < n; ++i) {
+      const Ref r = tensor_ref(params[i], "param", i);
+      if (!r.defined || r.dtype != RG_F32) throw std::invalid_argument("param[" + std::to_string(i) + "] must be a float32 tensor");
+      if (i == 0) device_ = r.device;
+      if (r.device != device_) throw std::invalid_argument("param[" + std::to_string(i) + "] is on another device");
+      p.push_back(r.ptr);
+      numel.push_back(r.numel);
+    }
+    for (size_t i = 0; i < n; ++i) {
+      const Ref r = tensor_ref(grads[i], "grad", i);
+      if (!r.defined || r.numel != numel[i] || r.device != device_)
+        throw std::invalid_argument("grad[" + std::to_string(i) + "] must be a tensor of its parameter's size and device");
+      g.push_back(r.ptr);
+      gdt.push_back(r.dtype);
+    }
+    column(state1, "state1", s1, nullptr, true);
+    column(state2, "state2", s2, nullptr, true);
+    column(copies, "model_copy", c, &cdt, false);
+    check(rg_optim_create(&opt_, device_, (int)n, p.data(), g.data(), s1.empty() && state1.is_none() ? nullptr : s1.data(),
+                          s2.empty() && state2.is_none() ? nullptr : s2.data(), copies.is_none() ? nullptr : c.data(),
+                          numel.data(), gdt.data(), copies.is_none() ? nullptr : cdt.data()));
+  }
+  ~Optim() { close(); }
+  Optim(const Optim&) = delete;
+  Optim& operator=(const Optim&) = delete;
+  void close() {
+    if (opt_ != nullptr) {
+      rg_optim_destroy(opt_);
+      opt_ = nullptr;
+    }
+  }
+  void adam_step(double lr, double beta1, double beta2, double eps, double weight_decay, int64_t step, bool decoupled,
+                 bool maximize, float grad_scale) {
+    rg_adam_args a{lr, beta1, beta2, eps, weight_decay, step, decoupled ? 1 : 0, maximize ? 1 : 0, grad_scale, nullptr};
+    check(rg_adam_step(handle(), &a, current_stream(device_)));
+  }
+  void sgd_step(double lr, double momentum, double dampening, double weight_decay, bool nesterov, bool maximize,
+                bool first_step, float grad_scale) {
+    rg_sgd_args a{lr, momentum, dampening, weight_decay, nesterov ? 1 : 0, maximize ? 1 : 0, first_step ? 1 : 0, grad_scale, nullptr};
+    check(rg_sgd_step(handle(), &a, current_stream(device_)));
+  }
+
+ private:
+  rg_optim* handle() {
+    if (opt_ == nullptr) throw std::runtime_error("the optimizer table is closed");
+    return opt_;
+  }
+  rg_optim* opt_ = nullptr;
+  int device_ = 0;
+  py::object keep_;  // the table points into these tensors
+};
+
 void copy_cast(const py::handle& dst, const py::handle& src, float scale) {
   const Ref d = tensor_ref(dst, "dst", 0);
   const Ref s = tensor_ref(src, "src", 0);
@@ -222,4 +301,15 @@ PYBIND11_MODULE(_ranncgrad, m) {
       .def_property_readonly("chunk_elems", &Plan::chunk_elems)
       .def_property_readonly("total_numel", &Plan::total_numel)
       .def_property_readonly("num_tensors", &Plan::num_tensors);
+  py::class_<Optim>(m, "Optim")
+      .def(py::init<const py::sequence&, const py::sequence&, const py::object&, const py::object&, const py::object&>(),
+           py::arg("params"), py::arg("grads"), py::arg("state1") = py::none(), py::arg("state2") = py::none(),
+           py::arg("model_copies") = py::none())
+      .def("adam_step", &Optim::adam_step, py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("eps"),
+           py::arg("weight_decay"), py::arg("step"), py::arg("decoupled") = false, py::arg("maximize") = false,
+           py::arg("grad_scale") = 1.0f)
+      .def("sgd_step", &Optim::sgd_step, py::arg("lr"), py::arg("momentum") = 0.0, py::arg("dampening") = 0.0,
+           py::arg("weight_decay") = 0.0, py::arg("nesterov") = false, py::arg("maximize") = false,
+           py::arg("first_step") = false, py::arg("grad_scale") = 1.0f)
+      .def("close", &Optim::close);
 }

@@ -69,3 +69,40 @@ def test_fused_step_through_pybind_matches_oracle_and_ctypes():
     pa.close()
     with pytest.raises(RuntimeError, match="closed"):
         pa.grad_norm()
+
+
+@pytest.mark.gpu
+def test_optimizer_table_through_pybind_matches_ctypes():
+    from rannc_amd import _lib
+    from rannc_amd.multi_tensor import stream_handle
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(6)
+    shapes = [(70001,), (33,), (4096,)]
+    p0 = [torch.randn(s, generator=g) for s in shapes]
+    grads = [(torch.randn(s, generator=g) * 1e-2).to(dev) for s in shapes]
+    sets = []
+    for _ in range(2):
+        sets.append(dict(p=[t.to(dev) for t in p0], m=[torch.zeros(s, device=dev) for s in shapes],
+                         v=[torch.zeros(s, device=dev) for s in shapes],
+                         c=[torch.zeros(s, device=dev, dtype=torch.bfloat16) for s in shapes]))
+    a, b = sets
+    oa = _ranncgrad.Optim(a["p"], grads, a["m"], a["v"], a["c"])
+    ob = _lib.OptimTable(0, [t.data_ptr() for t in b["p"]], [t.data_ptr() for t in grads], [t.data_ptr() for t in b["m"]],
+                         [t.data_ptr() for t in b["v"]], [t.data_ptr() for t in b["c"]], [t.numel() for t in p0],
+                         [_lib.RG_F32] * 3, [_lib.RG_BF16] * 3)
+    for step in (1, 2):
+        oa.adam_step(1e-3, 0.9, 0.999, 1e-8, 0.01, step)
+        ob.adam_step(1e-3, 0.9, 0.999, 1e-8, 0.01, step, stream=stream_handle(dev))
+    oa.sgd_step(0.1)
+    ob.sgd_step(0.1, stream=stream_handle(dev))
+    for k in "pmvc":
+        for x, y in zip(a[k], b[k]):
+            assert_bits_equal(x.cpu(), y.cpu(), f"pybind vs ctypes {k}")
+    assert not torch.equal(a["p"][0].cpu(), p0[0])
+    with pytest.raises(ValueError, match="float32"):
+        _ranncgrad.Optim([torch.zeros(4, device=dev, dtype=torch.float16)], [torch.zeros(4, device=dev)])
+    with pytest.raises(ValueError, match="exp_avg"):
+        _ranncgrad.Optim([torch.zeros(4, device=dev)], [torch.zeros(4, device=dev)]).adam_step(1e-3, 0.9, 0.999, 1e-8, 0.0, 1)
+    oa.close()
+    with pytest.raises(RuntimeError, match="closed"):
+        oa.sgd_step(0.1)
