@@ -222,10 +222,15 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   // The Infinity Cache holds 256 MiB: below that a second pass can still hit in cache.
   p->streaming = bytes > (int64_t)256 << 20;
   p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total);
+  // Tuning knobs, read once per plan (defaults are what measured best on MI355X):
+  //   RG_WRITE_TILE_ELEMS    elements per block of a writing pass (>= 256)
+  //   RG_XCD_REDUCE / _WRITE block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
+  //   RG_REDUCE_TILE_FACTOR  tile of a reducing + writing pass, in write tiles (0 = per operation)
   if (const char* env = getenv("RG_WRITE_TILE_ELEMS")) p->write_tile_elems = atoll(env);
   if (const char* env = getenv("RG_XCD_REDUCE")) p->xcd_reduce = atoi(env);
   if (const char* env = getenv("RG_XCD_WRITE")) p->xcd_write = atoi(env);
   if (const char* env = getenv("RG_REDUCE_TILE_FACTOR")) p->reduce_tile_factor = atoll(env);
+  if (p->reduce_tile_factor < 0) p->reduce_tile_factor = 0;
 
   p->chunk_begin.assign((size_t)n + 1, 0);
   for (int i = 0; i < n; ++i)
