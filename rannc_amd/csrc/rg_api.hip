@@ -37,12 +37,14 @@ struct rg_plan {
   bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
   int64_t write_tile_elems = kWriteTileElems;
   int xcd_reduce = 64;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
-  int xcd_write = 0;
+  int xcd_write = 0;                 //   ... when every source sits on the line grid of its destination
+  int xcd_write_offgrid = 256;       //   ... when some source does not (see fill_chunk_records)
   int64_t reduce_tile_factor = 0;    // tile of a reducing + writing pass, in write tiles (0 = per operation)
   float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
   std::vector<TensorDesc> host_tensors;
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
   bool dst_heads = false;            // some destination starts off a 128-byte boundary
+  bool offgrid = false;              // some source is off the 128-byte grid of its destination
 
   // one device allocation, carved up
   char* dev_base = nullptr;
@@ -88,11 +90,18 @@ static int64_t tensor_head(const void* src, const void* dst, int ss, int ds) {
 // the number of chunks stays ceil(numel / C) whatever the addresses are (trailing chunks may be empty).
 static void fill_chunk_records(rg_plan* p, ChunkRec* out) {
   p->dst_heads = false;
+  p->offgrid = false;
   for (int i = 0; i < p->n_tensors; ++i) {
     const TensorDesc& t = p->host_tensors[(size_t)i];
     const int ss = elem_size(t.src_dtype), ds = elem_size(t.dst_dtype);
     const int64_t head = tensor_head(t.src, t.dst, ss, ds);
     if (t.dst != nullptr && t.numel > 0 && head != 0) p->dst_heads = true;
+    // Write tiles start on destination lines; where the matching source address is not on a
+    // line too, the line at every tile boundary is read by two blocks.  Such plans give each
+    // XCD runs of consecutive tiles, so that the second read hits that XCD's L2.
+    if (t.dst != nullptr && t.src != nullptr && t.numel > head &&
+        ((reinterpret_cast<uintptr_t>(t.src) + (uintptr_t)(head * ss)) & (kAlignBytes - 1)) != 0)
+      p->offgrid = true;
     for (int64_t c = p->chunk_begin[(size_t)i]; c < p->chunk_begin[(size_t)i + 1]; ++c) {
       const int64_t j = c - p->chunk_begin[(size_t)i];
       const int64_t start = j == 0 ? 0 : std::min(t.numel, head + j * p->chunk_elems);
@@ -224,11 +233,12 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total);
   // Tuning knobs, read once per plan (defaults are what measured best on MI355X):
   //   RG_WRITE_TILE_ELEMS    elements per block of a writing pass (>= 256)
-  //   RG_XCD_REDUCE / _WRITE block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
+  //   RG_XCD_REDUCE / _WRITE block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run);
+  //                          unset, writing passes use 0, or runs of 256 when a source is off its destination's line grid
   //   RG_REDUCE_TILE_FACTOR  tile of a reducing + writing pass, in write tiles (0 = per operation)
   if (const char* env = getenv("RG_WRITE_TILE_ELEMS")) p->write_tile_elems = atoll(env);
   if (const char* env = getenv("RG_XCD_REDUCE")) p->xcd_reduce = atoi(env);
-  if (const char* env = getenv("RG_XCD_WRITE")) p->xcd_write = atoi(env);
+  if (const char* env = getenv("RG_XCD_WRITE")) p->xcd_write = p->xcd_write_offgrid = atoi(env);
   if (const char* env = getenv("RG_REDUCE_TILE_FACTOR")) p->reduce_tile_factor = atoll(env);
   if (p->reduce_tile_factor < 0) p->reduce_tile_factor = 0;
 
@@ -384,7 +394,7 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   a.tile_elems = (int32_t)p->chunk_elems;
   a.tiles_per_chunk = 1;
   a.peel_heads = p->dst_heads ? 1 : 0;
-  a.xcd_run = p->xcd_write;
+  a.xcd_run = p->offgrid ? p->xcd_write_offgrid : p->xcd_write;
   a.scale = scale;
   a.write_on_overflow = 0;
   a.zero_fill = 0;
@@ -484,7 +494,7 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
-  a.xcd_run = p->xcd_write;
+  a.xcd_run = p->offgrid ? p->xcd_write_offgrid : p->xcd_write;
   split_for_write(p, a);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, s));
   if (ev) RG_HIP(hipEventRecord(ev[3], s));
@@ -631,6 +641,9 @@ RG_API int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t nume
   a.single_chunk_elems = chunk;
   a.single_head = tensor_head(src_dev, dst_dev, ss, ds);
   a.peel_heads = a.single_head != 0 ? 1 : 0;
+  if (src_dev != nullptr && numel > a.single_head &&
+      ((reinterpret_cast<uintptr_t>(src_dev) + (uintptr_t)(a.single_head * ss)) & (kAlignBytes - 1)) != 0)
+    a.xcd_run = 256;   // source off the destination's line grid: consecutive tiles share an XCD's L2
   a.n_chunks = n_chunks;
   a.tile_elems = kWriteTileElems;
   a.tiles_per_chunk = (int32_t)tiles;
