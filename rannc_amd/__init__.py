@@ -164,6 +164,48 @@ class RaNNCModule(_pyrannc.RaNNCModule):
         p = self.get_param(name, amp_master_param)
         return p.grad
 
+    # ------------------------------------------------------------------ checkpoints
+    def state_dict(self, *args, no_hook=False, amp_master_params=True, rank0_only=True, **kwargs):
+        r"""
+        ``state_dict`` of the wrapped model (``pyrannc/__init__.py:401-436``): once deployed, one
+        entry per parameter name - parameters that share data appear under every one of their
+        names - holding the fp32 amp master when ``amp_master_params`` and amp are on.  Like the
+        reference it lists parameters only.  ``no_hook`` leaves out the model's state-dict hooks.
+        """
+        if not self.ready:
+            return self.model.state_dict(*args, **kwargs)
+        stashed = None
+        if no_hook:
+            stashed = {m: m._state_dict_hooks for m in self.model.modules()}
+            for m in stashed:
+                m._state_dict_hooks = type(m._state_dict_hooks)()
+        shared = {}
+        for n, p in self.model.named_parameters(remove_duplicate=False):
+            shared.setdefault(id(p), []).append(n)
+        new_state_dict = {}
+        try:
+            for n in self.model.state_dict(*args, **kwargs):
+                if n in self.name_to_param:
+                    param = self.get_param(n, amp_master_params and self.enable_apex_amp)
+                    for alias in shared.get(id(self.name_to_param[n]), [n]):
+                        new_state_dict[alias] = param
+        finally:
+            if stashed is not None:
+                for m, hooks in stashed.items():
+                    m._state_dict_hooks = hooks
+        return new_state_dict
+
+    def load_state_dict(self, *args, **kwargs):
+        r"""
+        Loads a ``state_dict`` into the wrapped model (``pyrannc/__init__.py:438-451``).  A deployed
+        module is undeployed first, so the next forward pass registers the new values.
+        """
+        if self.ready:
+            self.undeploy()
+            self.ready = False
+            self.amp_master_param_registered = False
+        return self.model.load_state_dict(*args, **kwargs)
+
     @property
     def use_amp_master_params_flag(self):
         return self.use_amp_master_params()

@@ -390,3 +390,44 @@ def test_clone_grad_summer_matches_the_reference_loop(dtype):
                 assert c.grad is None or bool((c.grad == 0).all())
     with pytest.raises(ValueError):
         CloneGradSummer([params[0]], [[params[1]]])
+
+
+def test_state_dict_returns_masters_under_every_shared_name_and_load_redeploys():
+    class Tied(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = torch.nn.Embedding(20, 16)
+            self.proj = torch.nn.Linear(16, 20, bias=False)
+            self.proj.weight = self.emb.weight                 # shared parameter, two names
+            self.register_buffer("steps", torch.zeros(1))
+
+        def forward(self, idx):
+            return self.proj(self.emb(idx))
+
+    torch.manual_seed(9)
+    model = Tied().to(DEV)
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    before = rm.state_dict()
+    assert "steps" in before                                    # not deployed yet: the model's own state_dict
+    idx = torch.randint(0, 20, (8,), device=DEV)
+    loss = rm(idx).float().pow(2).mean()
+    with amp.scale_loss(loss, opt) as scaled:
+        scaled.backward()
+    rm.clip_grad_norm(1.0)
+    opt.step()
+    sd = rm.state_dict()
+    assert set(sd.keys()) == {"emb.weight", "proj.weight"}      # parameters only, every alias
+    assert sd["emb.weight"] is sd["proj.weight"] and sd["emb.weight"].dtype == torch.float32
+    master = opt._amp_stash.all_fp32_from_fp16_params[0]
+    assert sd["emb.weight"].data_ptr() == master.data_ptr()
+    half = rm.state_dict(amp_master_params=False)
+    assert half["emb.weight"].dtype == torch.float16
+    assert_bits_equal(half["emb.weight"].cpu(), oracle.cast(master.detach().cpu(), torch.float16), "model copy of the master")
+    # loading undeploys; the next call deploys again with the loaded values
+    new_vals = {k: torch.full_like(v, 0.5) for k, v in model.state_dict().items()}
+    rm.load_state_dict(new_vals)
+    assert not rm.ready
+    rm(idx)
+    assert rm.ready and float(rm.get_param("emb.weight").detach().float().mean()) == 0.5
