@@ -63,6 +63,10 @@ class _AmpStash:
         # addresses, so the device table is built once
         self.master_grad_bucket: Optional[torch.Tensor] = None
         self.master_grad_views: List[torch.Tensor] = []
+        # fp32 parameters (batch norm under O2): tables for the in-place unscale of fresh
+        # gradients and for adding fresh gradients onto stashed ones (gradient accumulation)
+        self.fp32_unscale_plans = None
+        self.fp32_accumulate_plans = None
 
 
 class LossScaler:
@@ -252,6 +256,13 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
     scaler = _amp_state.loss_scalers[0]
     stash = optimizer._amp_stash
     _lazy_init_maybe_master_weights(optimizer)
+    # Gradients that fp32 parameters already hold are unscaled: set them aside so that the
+    # backward pass does not add scaled values onto them (Apex stashes them the same way).
+    stashed_fp32 = {}
+    for p in stash.all_fp32_from_fp32_params:
+        if p.grad is not None:
+            stashed_fp32[id(p)] = p.grad
+            p.grad = None
     yield loss.float() * scaler.loss_scale()
     model_grads, master_grads = [], []
     if stash.master_grad_bucket is None and stash.all_fp32_from_fp16_params:
@@ -283,14 +294,32 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
     if model_grads:
         scaler.unscale(stash, model_grads, master_grads, accumulate=accumulate)
     # fp32 parameters keep their own .grad; it carries the loss scale too
-    fp32_grads = [p.grad for p in stash.all_fp32_from_fp32_params if p.grad is not None]
-    if fp32_grads:
-        plan = TensorPlan(fp32_grads, fp32_grads)
-        with torch.no_grad():
-            plan.unscale_pack(1.0 / scaler.loss_scale())
-        if plan.result().overflow:
-            scaler._has_overflow = True
-        plan.close()
+    from ..param_storage import _PlanCache
+    if stash.fp32_unscale_plans is None:
+        stash.fp32_unscale_plans, stash.fp32_accumulate_plans = _PlanCache(), _PlanCache()
+    inv = 1.0 / scaler.loss_scale()
+    fresh32, new32, old32 = [], [], []
+    for p in stash.all_fp32_from_fp32_params:
+        kept = stashed_fp32.get(id(p))
+        if p.grad is None:
+            p.grad = kept                          # nothing new: the stashed gradient stays
+        elif kept is None:
+            fresh32.append(p.grad)
+        else:
+            new32.append(p.grad)
+            old32.append(kept)
+            p.grad = kept                          # kept += new * inv below
+    with torch.no_grad():
+        if fresh32:
+            plan = stash.fp32_unscale_plans.get(fresh32, fresh32)
+            plan.unscale_pack(inv)
+            if plan.result().overflow:
+                scaler._has_overflow = True
+        if new32:
+            plan = stash.fp32_accumulate_plans.get(new32, old32)
+            plan.unscale_accumulate(inv)
+            if plan.result().overflow:
+                scaler._has_overflow = True
     should_skip = scaler.update_scale()
     if should_skip:
         stash.skip_next_step = True

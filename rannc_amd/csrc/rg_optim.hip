@@ -67,6 +67,12 @@ constexpr int kOptThreads = RG_OPT_THREADS;
 constexpr int kOptTileElems = RG_OPT_TILE_ELEMS;
 constexpr int kOptE = 4;    // elements per lane per instruction
 constexpr int kOptU = RG_OPT_UNROLL;   // vectors per array a lane has in flight
+#ifndef RG_OPT_NT_LOAD
+#define RG_OPT_NT_LOAD 1
+#endif
+#ifndef RG_OPT_NT_STORE
+#define RG_OPT_NT_STORE 1
+#endif
 
 template <int ALGO>
 __device__ __forceinline__ void update_one(float& p, float g, float& s1, float& s2, const OptConst& c, float gscale) {
@@ -109,6 +115,7 @@ template <int ALGO, int G, int C, bool NT>
 __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int len, const OptConst& c, float gscale) {
   constexpr int T = kOptThreads;
   constexpr int E = kOptE;
+  constexpr bool NTL = NT && RG_OPT_NT_LOAD, NTS = NT && RG_OPT_NT_STORE;
   constexpr int GS = ElemSize<G>::value;
   constexpr bool kCopy = C >= 0;
   constexpr int CD = kCopy ? C : RG_F32;
@@ -144,12 +151,12 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
   }
 
   auto vec = [&](int e, Raw<RG_F32, E>& rp, Raw<G, E>& rg, Raw<RG_F32, E>& r1, Raw<RG_F32, E>& r2) {
-    rp = Mem<RG_F32, E, NT>::load(pp + (size_t)e * 4);
-    rg = Mem<G, E, NT>::load(gp + (size_t)e * GS);
+    rp = Mem<RG_F32, E, NTL>::load(pp + (size_t)e * 4);
+    rg = Mem<G, E, NTL>::load(gp + (size_t)e * GS);
     r1 = rp;
     r2 = rp;
-    if (use_s1) r1 = Mem<RG_F32, E, NT>::load(s1p + (size_t)e * 4);
-    if (ALGO == kAdam) r2 = Mem<RG_F32, E, NT>::load(s2p + (size_t)e * 4);
+    if (use_s1) r1 = Mem<RG_F32, E, NTL>::load(s1p + (size_t)e * 4);
+    if (ALGO == kAdam) r2 = Mem<RG_F32, E, NTL>::load(s2p + (size_t)e * 4);
   };
   auto finish = [&](int e, const Raw<RG_F32, E>& rp, const Raw<G, E>& rg, const Raw<RG_F32, E>& r1, const Raw<RG_F32, E>& r2) {
     float p[E], g[E], s1[E], s2[E];
@@ -159,10 +166,10 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
     Codec<RG_F32, E>::unpack(r2, s2);
 #pragma unroll
     for (int j = 0; j < E; ++j) update_one<ALGO>(p[j], g[j], s1[j], s2[j], c, gscale);
-    Mem<RG_F32, E, NT>::store(pp + (size_t)e * 4, Codec<RG_F32, E>::pack(p));
-    if (use_s1) Mem<RG_F32, E, NT>::store(s1p + (size_t)e * 4, Codec<RG_F32, E>::pack(s1));
-    if (ALGO == kAdam) Mem<RG_F32, E, NT>::store(s2p + (size_t)e * 4, Codec<RG_F32, E>::pack(s2));
-    if constexpr (kCopy) Mem<CD, E, NT>::store(cp + (size_t)e * CS, Codec<CD, E>::pack(p));
+    Mem<RG_F32, E, NTS>::store(pp + (size_t)e * 4, Codec<RG_F32, E>::pack(p));
+    if (use_s1) Mem<RG_F32, E, NTS>::store(s1p + (size_t)e * 4, Codec<RG_F32, E>::pack(s1));
+    if (ALGO == kAdam) Mem<RG_F32, E, NTS>::store(s2p + (size_t)e * 4, Codec<RG_F32, E>::pack(s2));
+    if constexpr (kCopy) Mem<CD, E, NTS>::store(cp + (size_t)e * CS, Codec<CD, E>::pack(p));
   };
   constexpr int U = kOptU;
   constexpr int kIter = T * E * U;

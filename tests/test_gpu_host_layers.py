@@ -431,3 +431,27 @@ def test_state_dict_returns_masters_under_every_shared_name_and_load_redeploys()
     assert not rm.ready
     rm(idx)
     assert rm.ready and float(rm.get_param("emb.weight").detach().float().mean()) == 0.5
+
+
+def test_amp_accumulates_fp32_parameter_gradients_too():
+    # batch norm stays fp32 under O2: its gradients live on the model parameter and must
+    # accumulate as  grad = grad + new_scaled_grad * inv_scale  over scale_loss contexts
+    torch.manual_seed(4)
+    model = torch.nn.Sequential(torch.nn.Linear(16, 24), torch.nn.BatchNorm1d(24), torch.nn.Linear(24, 4)).to(DEV)
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8)
+    assert model[1].weight.dtype == torch.float32 and model[0].weight.dtype == torch.float16
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    want_w = None
+    for it in range(3):
+        x = torch.randn(32, 16, device=DEV, dtype=torch.float16)
+        loss = rm(x).float().pow(2).mean()
+        with amp.scale_loss(loss, opt) as scaled:
+            scaled.backward()
+            scaled_grad = model[1].weight.grad.detach().cpu().clone()    # what this backward produced, still scaled
+        if want_w is None:
+            want_w, _ = oracle.unscale_and_check([scaled_grad], 1.0 / 256.0)
+        else:
+            oracle.unscale_accumulate(want_w, [scaled_grad], 1.0 / 256.0)
+        assert_bits_equal(model[1].weight.grad.cpu(), want_w[0], f"bn weight grad after {it + 1} micro-batches")
+    opt.step()
