@@ -328,9 +328,10 @@ class ParamStorage:
         for d in (self._clip_plans, self._scale_plans):
             for k in [k for k in d if k[0] == graph_id]:
                 d.pop(k).clear()
-        for d in (self._zero_plans, self._stage_plans):
-            if graph_id in d:
-                d.pop(graph_id).clear()
+        if graph_id in self._zero_plans:
+            self._zero_plans.pop(graph_id).clear()
+        for k in [k for k in self._stage_plans if k.split("/")[0] == graph_id]:
+            self._stage_plans.pop(k).clear()
 
     # ------------------------------------------------------------------ per-step operations
     def prepare_backward(self, graph_id: str) -> None:
@@ -450,9 +451,10 @@ class ParamStorage:
             back_dst.append(grad.view(-1))
             bufs.append(buf)
         if srcs:
+            # the caching allocator usually hands back last step's addresses: the tables are reused
             with torch.no_grad():
-                TensorPlan(srcs, dsts).scale_cast(1.0)
-                TensorPlan(back_src, back_dst).scale_cast(1.0)
+                self._stage_plans.setdefault(graph_id + "/pack", _PlanCache()).get(srcs, dsts).scale_cast(1.0)
+                self._stage_plans.setdefault(graph_id + "/back", _PlanCache()).get(back_src, back_dst).scale_cast(1.0)
         return bufs
 
     def bcast_params_zero(self, graph_id: str, grad: bool = False) -> None:
