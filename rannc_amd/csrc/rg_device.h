@@ -27,15 +27,24 @@ template <> struct Raw<RG_BF16, 4> { u32x2 v; };
 template <> struct Raw<RG_F16, 8> { u32x4 v; };
 template <> struct Raw<RG_BF16, 8> { u32x4 v; };
 
+// Every pointer these helpers see addresses device (global) memory; pointers read from a
+// table in memory are "generic" to the compiler, which would then emit flat_* instructions
+// (slower to issue, and they tie up the LDS counter).  The casts below state the address
+// space, so the accesses compile to global_* whatever the compiler could infer.
+#define RG_GLOBAL __attribute__((address_space(1)))
+
 // Loads at element alignment.
 template <bool NT> __device__ __forceinline__ u32x4 ld16_a4(const char* p) {
-  return NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4_a4*>(p)) : *reinterpret_cast<const u32x4_a4*>(p);
+  const RG_GLOBAL u32x4_a4* g = (const RG_GLOBAL u32x4_a4*)p;
+  return NT ? __builtin_nontemporal_load(g) : *g;
 }
 template <bool NT> __device__ __forceinline__ u32x4 ld16_a2(const char* p) {
-  return NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4_a2*>(p)) : *reinterpret_cast<const u32x4_a2*>(p);
+  const RG_GLOBAL u32x4_a2* g = (const RG_GLOBAL u32x4_a2*)p;
+  return NT ? __builtin_nontemporal_load(g) : *g;
 }
 template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
-  return NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x2_a2*>(p)) : *reinterpret_cast<const u32x2_a2*>(p);
+  const RG_GLOBAL u32x2_a2* g = (const RG_GLOBAL u32x2_a2*)p;
+  return NT ? __builtin_nontemporal_load(g) : *g;
 }
 // Stores: the pointer type promises element alignment only (what the peel guarantees beyond
 // that is a performance matter, not a correctness one).
@@ -43,12 +52,14 @@ template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
 #define RG_NT_STORES 1
 #endif
 template <bool NT> __device__ __forceinline__ void st16(char* p, u32x4 v) {
-  if (NT && RG_NT_STORES) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_a2*>(p));
-  else *reinterpret_cast<u32x4_a2*>(p) = v;
+  RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
+  if (NT && RG_NT_STORES) __builtin_nontemporal_store(v, g);
+  else *g = v;
 }
 template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
-  if (NT && RG_NT_STORES) __builtin_nontemporal_store(v, reinterpret_cast<u32x2_a2*>(p));
-  else *reinterpret_cast<u32x2_a2*>(p) = v;
+  RG_GLOBAL u32x2_a2* g = (RG_GLOBAL u32x2_a2*)p;
+  if (NT && RG_NT_STORES) __builtin_nontemporal_store(v, g);
+  else *g = v;
 }
 
 template <int DT, int E, bool NT> struct Mem;
