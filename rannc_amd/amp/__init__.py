@@ -57,7 +57,6 @@ class _AmpStash:
         self.pending_finish = False        # fused mode: the write pass has not run yet
         self.fused = False
         self.last_result = None            # rg_step_result of the last unscale
-        self.norm_is_fresh = False
         # packed fp32 bucket the master gradients are views of (the reference's
         # consolidated_master_grads_, src/comp/ParamStorage.cpp:68-70, 92-97): stable
         # addresses, so the device table is built once
@@ -112,7 +111,6 @@ class LossScaler:
             else:
                 stash.unscale_plan.unscale_pack(inv)
         stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
-        stash.norm_is_fresh = True
         if stash.last_result.overflow:
             self._has_overflow = True
 
@@ -210,7 +208,6 @@ def finish_unscale(optimizer: torch.optim.Optimizer, max_norm: float = 0.0) -> N
         with torch.no_grad():
             stash.unscale_plan.step_finish(float(max_norm))
         stash.pending_finish = False
-        stash.norm_is_fresh = False
 
 
 def _master_to_model(optimizer: torch.optim.Optimizer) -> None:
@@ -241,7 +238,6 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
         ret = old_step(*args, **kwargs)
         if not getattr(stash, "optimizer_copies_back", False):
             _master_to_model(optimizer)
-        stash.norm_is_fresh = False
         return ret
 
     optimizer.step = new_step
