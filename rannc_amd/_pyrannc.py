@@ -8,7 +8,7 @@ failures raise ``RuntimeError``.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional, Tuple
+from typing import Dict, Tuple
 
 import torch
 

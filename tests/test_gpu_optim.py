@@ -2,8 +2,6 @@
 torch.optim bit for bit).  Floating point: parameter and moments must agree with the oracle
 to 2e-6 relative (plus 2e-6 of the learning rate for parameters near zero - an update is at
 most about lr); the model copy must be the bit-exact rounding of the GPU's own parameter."""
-import math
-
 import pytest
 import torch
 
