@@ -24,6 +24,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # FETCH_SIZE / WRITE_SIZE runs of this same command, each scaled by what the counter reads for
 # a plain 1 GiB copy (profiles/fused_step_c2_bert_large_hbm_traffic.txt).  Missing = not measured.
 MEASURED_TRAFFIC_BYTES = {"c2_bert_large": 2021550504}
+# the Adam step with bf16 model copy, same method (profiles/adam_step_c2_bert_large_kernel_stats.txt)
+MEASURED_TRAFFIC_BYTES_ADAM = {"c2_bert_large": 10075311450}
 
 
 def parse_args():
@@ -163,7 +165,8 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
                    "bytes_per_elem": bytes_per_elem, "model_copy_dtype": str(copy_dt), "seed": args.seed},
         "pct_of_hbm_peak": round(100.0 * step_bytes / step_s / 1e9 / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "kernel": f"optim_kernel<{args.op}, streaming>", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES_ADAM.get(cfg.key) if adam else None,
                      "algorithmic_bytes_per_launch": step_bytes, "avg_launch_ms": round(launch_ms, 4)},
     }
     table.close()
