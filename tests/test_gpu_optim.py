@@ -227,3 +227,47 @@ def test_bad_arguments_are_value_errors():
         q = torch.zeros(4, device=DEV, dtype=torch.bfloat16, requires_grad=True)
         q.grad = torch.zeros_like(q)
         FusedAdam([q]).step()
+
+
+def test_whole_step_fused_unscale_clip_then_fused_adam():
+    """scale_loss (read pass) -> clip_grad_norm (write pass, clipped) -> FusedAdam.step (masters +
+    model copies), against the oracle's sequence unscale -> norm -> clip -> Adam -> half(master)."""
+    torch.manual_seed(11)
+    half = torch.bfloat16
+    model = torch.nn.Sequential(torch.nn.Linear(64, 96), torch.nn.Tanh(), torch.nn.Linear(96, 10)).to(DEV)
+    opt = FusedAdam(model.parameters(), lr=5e-3, weight_decay=0.01)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 10, half_dtype=half, fused=True)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    ms = vs = None
+    for it in range(3):
+        x = torch.randn(32, 64, device=DEV, dtype=half)
+        loss = rm(x).float().pow(2).sum()
+        with amp.scale_loss(loss, opt) as scaled:
+            scaled.backward()
+            model_grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
+        stash = opt._amp_stash
+        masters = stash.all_fp32_from_fp16_params
+        scale = 2.0 ** 10
+        rm.clip_grad_norm(0.5)
+        want = oracle.fused_step(model_grads, ["f32"] * len(model_grads), 1.0 / scale, 0.5)
+        assert want.coef is not None, "the test is meant to clip"
+        offs = 0
+        want_grads = []
+        for m in masters:
+            want_grads.append(want.buckets["f32"][offs:offs + m.numel()].view(m.shape))
+            offs += m.numel()
+        for m, w in zip(masters, want_grads):
+            torch.testing.assert_close(m.grad.cpu(), w, rtol=2e-6, atol=0.0)      # coef agrees to 1e-6, values follow
+        m_cpu = [m.detach().cpu().clone() for m in masters]
+        g_cpu = [m.grad.detach().cpu().clone() for m in masters]
+        if ms is None:
+            ms = [torch.zeros_like(t) for t in m_cpu]
+            vs = [torch.zeros_like(t) for t in m_cpu]
+        opt.step()
+        oracle_optim.adam_step(m_cpu, g_cpu, ms, vs, it + 1, lr=5e-3, weight_decay=0.01)
+        for m, w, p in zip(masters, m_cpu, stash.all_fp16_params):
+            close(m, w, 5e-3 * RTOL, f"master it {it}")
+            assert_bits_equal(p.detach().cpu(), oracle_optim.model_copy(m.detach().cpu(), half), "model copy")
+        for a, b, m in zip(ms, vs, masters):
+            a.copy_(opt.state[m]["exp_avg"]); b.copy_(opt.state[m]["exp_avg_sq"])
+        opt.zero_grad()          # master gradients go back to None: the next unscale overwrites (else it accumulates)
