@@ -24,6 +24,7 @@ class _FusedBase(torch.optim.Optimizer):
         super().__init__(params, defaults)
         self._tables: Dict[Tuple, Tuple[_lib.OptimTable, Tuple, List]] = {}
         self._model_copies: Dict[int, torch.Tensor] = {}
+        self._steps: Dict[int, Tuple[torch.Tensor, int]] = {}     # id(param) -> (its step tensor, value)
         #: device pointer of an ``rg_step_result`` (``TensorPlan.plan.result_device_ptr()``): the step
         #: multiplies the gradients by its clip coefficient and does nothing when it says "skipped"
         self.gate: int = 0
@@ -95,6 +96,7 @@ class FusedAdam(_FusedBase):
                 loss = closure()
         for gi, group in enumerate(self.param_groups):
             by_step: Dict[int, List[torch.Tensor]] = {}
+            step_tensors = []
             for p in group["params"]:
                 if p.grad is None:
                     continue
@@ -104,8 +106,16 @@ class FusedAdam(_FusedBase):
                     st["step"] = torch.tensor(0.0, dtype=torch.float32)
                     st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                     st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
-                st["step"] += 1
-                by_step.setdefault(int(st["step"]), []).append(p)
+                # ``step`` stays a tensor (torch.optim's state layout); its integer value is mirrored
+                # here so that a step costs one batched increment instead of one tensor op per parameter
+                t = st["step"]
+                seen = self._steps.get(id(p))
+                count = (seen[1] if seen is not None and seen[0] is t else int(t)) + 1
+                self._steps[id(p)] = (t, count)
+                step_tensors.append(t)
+                by_step.setdefault(count, []).append(p)
+            if step_tensors:
+                torch._foreach_add_(step_tensors, 1)
             for step, ps in by_step.items():
                 ms = [self.state[p]["exp_avg"] for p in ps]
                 vs = [self.state[p]["exp_avg_sq"] for p in ps]
