@@ -34,8 +34,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_bert_large")
-    ap.add_argument("--op", default="fused_step", choices=["fused_step", "adam", "sgd"],
-                    help="fused_step (default: the graded metric) or the optimizer step that follows it")
+    ap.add_argument("--op", default="fused_step", choices=["fused_step", "adam", "sgd", "adam_from_model_grads"],
+                    help="fused_step (default: the graded metric), the optimizer step that follows it, or both "
+                         "without ever writing the unscaled gradients (read pass + clip decision + Adam reading the scaled grads)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--chunk-elems", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -108,10 +109,13 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
     from rannc_amd.multi_tensor import stream_handle
     from rannc_amd.workloads import make_grads
 
+    from rannc_amd.multi_tensor import TensorPlan
     grads, _ = make_grads(cfg, args.seed, device=str(dev))
     shapes = [g.shape for g in grads]
     copy_dt = grads[0].dtype if grads[0].dtype != torch.float32 else torch.bfloat16
-    del grads
+    direct = args.op == "adam_from_model_grads"
+    if not direct:
+        del grads
     n = sum(torch.Size(sh).numel() for sh in shapes)
     gen = torch.Generator(device=dev).manual_seed(args.seed)
     bucket = torch.randn(n, device=dev, generator=gen) * 1e-2
@@ -121,21 +125,29 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
         gviews.append(bucket.narrow(0, off, k))
         off += k
     params = [torch.randn(sh, device=dev, generator=gen) for sh in shapes]
-    adam = args.op == "adam"
+    adam = args.op in ("adam", "adam_from_model_grads")
     m = [torch.zeros_like(p) for p in params] if adam else None
     v = [torch.zeros_like(p) for p in params] if adam else None
     copies = [torch.zeros(sh, device=dev, dtype=copy_dt) for sh in shapes]
     code = {torch.float16: _lib.RG_F16, torch.bfloat16: _lib.RG_BF16}[copy_dt]
-    table = _lib.OptimTable(0, [t.data_ptr() for t in params], [t.data_ptr() for t in gviews],
+    gsrc = grads if direct else gviews
+    gcode = {torch.float32: _lib.RG_F32, torch.float16: _lib.RG_F16, torch.bfloat16: _lib.RG_BF16}[gsrc[0].dtype]
+    table = _lib.OptimTable(0, [t.data_ptr() for t in params], [t.data_ptr() for t in gsrc],
                             [t.data_ptr() for t in m] if adam else None, [t.data_ptr() for t in v] if adam else None,
-                            [t.data_ptr() for t in copies], [t.numel() for t in params], [_lib.RG_F32] * len(params),
+                            [t.data_ptr() for t in copies], [t.numel() for t in params], [gcode] * len(params),
                             [code] * len(params))
     st = stream_handle(dev)
     count = [0]
+    plan = TensorPlan(grads, gviews) if direct else None
+    gate = plan.plan.result_device_ptr() if direct else 0
 
     def step():
         count[0] += 1
-        if adam:
+        if direct:       # read pass (flag + norm), clip decision, Adam on the scaled gradients: nothing else is written
+            plan.step_begin(cfg.inv_scale)
+            plan.step_decide(cfg.max_norm)
+            table.adam_step(1e-3, 0.9, 0.999, 1e-8, 0.0, count[0], grad_scale=cfg.inv_scale, gate=gate, stream=st)
+        elif adam:
             table.adam_step(1e-3, 0.9, 0.999, 1e-8, 0.0, count[0], stream=st)
         else:
             table.sgd_step(0.01, stream=st)
@@ -152,7 +164,11 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     launch_ms = e0.elapsed_time(e1) / args.steps
-    bytes_per_elem = (16 + 12 + 2) if adam else (8 + 4 + 2)
+    gs = gsrc[0].element_size()
+    if direct:
+        bytes_per_elem = gs + (gs + 12) + 12 + 2      # read pass + Adam (grad, p, m, v in; p, m, v, copy out)
+    else:
+        bytes_per_elem = (16 + 12 + 2) if adam else (8 + 4 + 2)
     step_bytes = bytes_per_elem * n
     step_s = elapsed / args.steps
     achieved = step_bytes / (launch_ms * 1e-3) / 1e9
@@ -164,16 +180,23 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
         "config": {"workload": cfg.key, "op": args.op, "tensors": len(params), "elements": n,
                    "bytes_per_elem": bytes_per_elem, "model_copy_dtype": str(copy_dt), "seed": args.seed},
         "pct_of_hbm_peak": round(100.0 * step_bytes / step_s / 1e9 / HBM_PEAK_GBPS, 2),
-        "roofline": {"bound": "hbm", "kernel": f"optim_kernel<{args.op}, streaming>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": ("pass_kernel<reduce> + finalize + optim_kernel<adam>, all launches of a step"
+                                                 if direct else f"optim_kernel<{args.op}, streaming>"),
+                     "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES_ADAM.get(cfg.key) if adam else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES_ADAM.get(cfg.key) if args.op == "adam" else None,
                      "algorithmic_bytes_per_launch": step_bytes, "avg_launch_ms": round(launch_ms, 4)},
     }
     table.close()
+    if plan is not None:
+        res = plan.result()
+        out["config"].update({"clipped": bool(res.clipped), "overflow": int(res.overflow), "norm": res.norm})
+        plan.close()
     del params, m, v, copies, bucket, gviews
     torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_optimizer(args.op, shapes, args.seed, args.cpu_seconds, bytes_per_elem)
+        out["cpu_baseline"] = cpu_baseline_optimizer("adam" if adam else "sgd", shapes, args.seed, args.cpu_seconds,
+                                                     bytes_per_elem)
     return out
 
 

@@ -141,6 +141,13 @@ int rg_fused_step(rg_plan* plan, float inv_scale, float max_norm, int flags, voi
  * Together they move exactly the bytes of rg_fused_step. */
 int rg_step_begin(rg_plan* plan, float inv_scale, void* stream);
 int rg_step_finish(rg_plan* plan, float max_norm, int flags, void* stream);
+/* The clip decision alone: from the sums rg_step_begin left on the device, fills coef /
+ * clipped / skipped of the result block for max_norm and launches no pass over the
+ * gradients.  For callers whose next kernel consumes the decision on the device - the
+ * optimizer step below with `gate`, reading the still-scaled gradients with grad_scale =
+ * inv_scale - so that the unscaled, clipped gradients are never written to memory at all.
+ * The begin stays pending: rg_step_finish may still be called to write them. */
+int rg_step_decide(rg_plan* plan, float max_norm, int flags, void* stream);
 
 /* One pass: dst = round_dst(float(x) * inv_scale), overflow flag and norm as above, no
  * clip.  Apex multi_tensor_scale semantics (LossScaler.unscale). */
@@ -217,7 +224,8 @@ int rg_optim_destroy(rg_optim* opt);
 
 /* Arithmetic of torch.optim.Adam / AdamW (single-tensor form, amsgrad off), in fp32 with
  * the scalar factors computed in double and rounded once, as ATen does with Python scalars:
- *   g  = grad * grad_scale            (and * gate->coef; the whole step is skipped when gate->skipped)
+ *   g  = grad * grad_scale            (then * gate->coef, a second multiply, exactly what rg_step_finish
+ *                                      would have stored; the whole step is skipped when gate->skipped)
  *   g  = -g                           if maximize
  *   p  = p * (1 - lr * wd)            if decoupled_weight_decay (AdamW), else g = g + wd * p
  *   m  = m + (1 - beta1) * (g - m)

@@ -122,17 +122,23 @@ class RaNNCModule(_pyrannc.RaNNCModule):
         Clips gradients by their global L2 norm (``pyrannc/__init__.py:381-394``): iff
         ``norm + 1e-6 > max_grad_norm`` every gradient is multiplied by
         ``max_grad_norm / (norm + 1e-6)``.  With amp in fused mode the pending unscale is
-        completed and clipped in the same pass over the gradients.
+        completed and clipped in the same pass over the gradients; with a fused optimizer on
+        top only the decision is taken here and the optimizer's step kernel applies it.
         """
         if not self.ready:
             self._deploy()
         if self.enable_apex_amp:
             self._setup_amp_params()
             stash = getattr(self.optimizer, "_amp_stash", None)
-            if stash is not None and stash.pending_finish and not stash.all_fp32_from_fp32_params:
-                from .amp import finish_unscale
-                finish_unscale(self.optimizer, float(torch.tensor(max_grad_norm, dtype=torch.float32)))
-                return
+            max_f = float(torch.tensor(max_grad_norm, dtype=torch.float32))      # crosses the binding as a C float
+            if stash is not None and stash.pending_finish:
+                from .amp import can_step_from_model_grads, decide_clip, finish_unscale
+                if can_step_from_model_grads(self.optimizer):
+                    decide_clip(self.optimizer, max_f)      # the optimizer's step kernel applies it
+                    return
+                if not any(p.grad is not None for p in stash.all_fp32_from_fp32_params):
+                    finish_unscale(self.optimizer, max_f)
+                    return
             if stash is not None and stash.pending_finish:
                 from .amp import finish_unscale
                 finish_unscale(self.optimizer)
@@ -161,6 +167,10 @@ class RaNNCModule(_pyrannc.RaNNCModule):
         return super().get_param(self.name_to_pid[name], amp_master_param)
 
     def get_param_grad(self, name, amp_master_param=False):
+        stash = getattr(self.optimizer, "_amp_stash", None)
+        if amp_master_param and stash is not None and stash.pending_finish:
+            from .amp import finish_unscale
+            finish_unscale(self.optimizer)        # the master gradients are about to be looked at: write them
         p = self.get_param(name, amp_master_param)
         return p.grad
 

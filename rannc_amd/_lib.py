@@ -58,6 +58,7 @@ SIGNATURES = {
     "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
     "rg_step_begin": (_i, [_vp, _f, _vp]),
     "rg_step_finish": (_i, [_vp, _f, _i, _vp]),
+    "rg_step_decide": (_i, [_vp, _f, _i, _vp]),
     "rg_unscale_pack": (_i, [_vp, _f, _vp]),
     "rg_accumulate": (_i, [_vp, _f, _vp]),
     "rg_unscale_accumulate": (_i, [_vp, _f, _vp]),
@@ -208,6 +209,9 @@ class Plan:
 
     def step_finish(self, max_norm: float, flags: int = RG_STEP_DEFAULT, stream: int = 0) -> None:
         check(lib.rg_step_finish(self._handle, max_norm, flags, _vp(stream)))
+
+    def step_decide(self, max_norm: float, flags: int = RG_STEP_DEFAULT, stream: int = 0) -> None:
+        check(lib.rg_step_decide(self._handle, max_norm, flags, _vp(stream)))
 
     def unscale_pack(self, inv_scale: float, stream: int = 0) -> None:
         check(lib.rg_unscale_pack(self._handle, inv_scale, _vp(stream)))

@@ -55,6 +55,10 @@ class _AmpStash:
         self.unscale_key: Optional[tuple] = None
         self.copy_back_plan: Optional[TensorPlan] = None
         self.pending_finish = False        # fused mode: the write pass has not run yet
+        self.pending_inv_scale = 1.0       #   ... the 1/loss_scale its read pass ran with
+        self.pending_masters: List[torch.Tensor] = []      #   ... the masters and model gradients it covers
+        self.pending_model_grads: List[torch.Tensor] = []
+        self.decided_max_norm: Optional[float] = None      # clip_grad_norm asked for while the write is pending
         self.fused = False
         self.last_result = None            # rg_step_result of the last unscale
         # packed fp32 bucket the master gradients are views of (the reference's
@@ -108,6 +112,8 @@ class LossScaler:
             elif stash.fused:
                 stash.unscale_plan.step_begin(inv)
                 stash.pending_finish = True
+                stash.pending_inv_scale = inv
+                stash.decided_max_norm = None
             else:
                 stash.unscale_plan.unscale_pack(inv)
         stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
@@ -142,7 +148,13 @@ def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_lev
 
     ``fused=True`` defers the write of the unscaled master gradients from the ``scale_loss``
     exit to the next ``clip_grad_norm`` / ``optimizer.step``, so that unscale, norm, clip and
-    pack move ``(2s + d)`` bytes per element; until then master ``.grad`` holds stale data."""
+    pack move ``(2s + d)`` bytes per element; until then master ``.grad`` holds stale data.
+    When the optimizer is one of ``rannc_amd.fused_optim`` (and every stepped parameter is half
+    precision) the write never happens: ``clip_grad_norm`` only takes the clip decision on the
+    device and ``optimizer.step`` reads the scaled model gradients, applies ``1/scale`` and the
+    clip coefficient, updates the masters and writes the model copies in one kernel.  Anything
+    that looks at master gradients first (``calc_grad_norm``, ``get_param_grad``,
+    ``finish_unscale``) writes them, and the step then takes them from memory."""
     if opt_level != "O2":
         raise ValueError("only opt_level='O2' (fp32 masters for half parameters) is provided")
     bn = torch.nn.modules.batchnorm._BatchNorm
@@ -201,13 +213,36 @@ def master_params(optimizer: torch.optim.Optimizer) -> Iterator[torch.Tensor]:
             yield p
 
 
-def finish_unscale(optimizer: torch.optim.Optimizer, max_norm: float = 0.0) -> None:
-    """Fused mode: run the deferred write pass (clip to ``max_norm`` when > 0)."""
+def finish_unscale(optimizer: torch.optim.Optimizer, max_norm: Optional[float] = None) -> None:
+    """Fused mode: run the deferred write pass (clip to ``max_norm`` when > 0; by default to the
+    value an earlier ``decide_clip`` recorded, else no clipping)."""
     stash = optimizer._amp_stash
     if stash.pending_finish:
+        if max_norm is None:
+            max_norm = stash.decided_max_norm or 0.0
         with torch.no_grad():
             stash.unscale_plan.step_finish(float(max_norm))
         stash.pending_finish = False
+        stash.decided_max_norm = None
+
+
+def can_step_from_model_grads(optimizer: torch.optim.Optimizer) -> bool:
+    """True while the unscaled gradients need not be written at all: the write pass is still
+    pending, the optimizer is one whose step kernel can read the model gradients and the clip
+    decision itself, and every parameter it steps on has a half-precision model gradient (fp32
+    parameters are unscaled in place and would be missing from the norm)."""
+    stash = optimizer._amp_stash
+    return bool(stash.pending_finish and getattr(optimizer, "reads_grad_sources", False)
+                and not any(p.grad is not None for p in stash.all_fp32_from_fp32_params))
+
+
+def decide_clip(optimizer: torch.optim.Optimizer, max_norm: float) -> None:
+    """Fused mode with a fused optimizer: take the clip decision on the device (no pass over the
+    gradients); the optimizer's step kernel applies it while reading the model gradients."""
+    stash = optimizer._amp_stash
+    with torch.no_grad():
+        stash.unscale_plan.step_decide(float(max_norm))
+    stash.decided_max_norm = float(max_norm)
 
 
 def _master_to_model(optimizer: torch.optim.Optimizer) -> None:
@@ -234,6 +269,22 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
             stash.skip_next_step = False
             stash.pending_finish = False
             return None
+        if can_step_from_model_grads(optimizer) and not (args or kwargs):
+            # unscale, clip, update and model copy in one kernel: the step reads the still-scaled
+            # model gradients and the clip decision from the device
+            if stash.decided_max_norm is None:
+                decide_clip(optimizer, 0.0)
+            optimizer.set_grad_sources(stash.pending_masters, stash.pending_model_grads)
+            optimizer.grad_scale = stash.pending_inv_scale
+            optimizer.gate = stash.unscale_plan.plan.result_device_ptr()
+            try:
+                ret = old_step()
+            finally:
+                optimizer.set_grad_sources([], [])
+                optimizer.grad_scale, optimizer.gate = 1.0, 0
+            stash.pending_finish = False
+            stash.decided_max_norm = None
+            return ret
         finish_unscale(optimizer)
         ret = old_step(*args, **kwargs)
         if not getattr(stash, "optimizer_copies_back", False):
@@ -280,12 +331,15 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
             m = stash.all_fp32_from_fp16_params[i]
             m.grad = stash.master_grad_views[i]
             fill_zero_(m.grad.view(-1)) if m.grad.is_contiguous() else m.grad.zero_()
+    masters = []
     for i in sorted(fresh + live):
         p, m = stash.all_fp16_params[i], stash.all_fp32_from_fp16_params[i]
         if m.grad is None:
             m.grad = stash.master_grad_views[i]
         model_grads.append(p.grad)
         master_grads.append(m.grad)
+        masters.append(m)
+    stash.pending_masters, stash.pending_model_grads = masters, list(model_grads)
     scaler.clear_overflow_state()
     if model_grads:
         scaler.unscale(stash, model_grads, master_grads, accumulate=accumulate)

@@ -537,6 +537,19 @@ RG_API int rg_step_finish(rg_plan* p, float max_norm, int flags, void* stream) {
   return RG_OK;
 }
 
+RG_API int rg_step_decide(rg_plan* p, float max_norm, int flags, void* stream) {
+  const int rc = check_plan(p, kNeedSrc, "rg_step_decide");
+  if (rc != RG_OK) return rc;
+  if (p->begun_inv_scale == 0.0f) {
+    set_error("rg_step_decide: no rg_step_begin is pending on this plan");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  RG_HIP(launch_finalize_total(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0),
+                               reinterpret_cast<hipStream_t>(stream)));
+  return RG_OK;   // the begin stays pending: rg_step_finish may still write the gradients
+}
+
 RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_unscale_pack");
   if (rc != RG_OK) return rc;

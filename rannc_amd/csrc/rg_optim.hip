@@ -75,8 +75,11 @@ constexpr int kOptU = RG_OPT_UNROLL;   // vectors per array a lane has in flight
 #endif
 
 template <int ALGO>
-__device__ __forceinline__ void update_one(float& p, float g, float& s1, float& s2, const OptConst& c, float gscale) {
-  g = g * gscale;
+__device__ __forceinline__ void update_one(float& p, float g, float& s1, float& s2, const OptConst& c, float coef) {
+  // two multiplies, each rounded: the value a pass that wrote the unscaled, clipped gradient
+  // would have stored (x * 1 is x, so neither needs a branch)
+  g = g * c.grad_scale;
+  g = g * coef;
   if (c.maximize) g = -g;
   if (ALGO == kAdam) {
     p = p * c.param_mul;                                          // x * 1 is x: no branch needed
@@ -112,7 +115,7 @@ template <> __device__ __forceinline__ float load1<RG_BF16>(const char* p) {
 
 // One tile of one chunk.  G: gradient dtype; C: model-copy dtype, or -1 for none.
 template <int ALGO, int G, int C, bool NT>
-__device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int len, const OptConst& c, float gscale) {
+__device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int len, const OptConst& c, float coef) {
   constexpr int T = kOptThreads;
   constexpr int E = kOptE;
   constexpr bool NTL = NT && RG_OPT_NT_LOAD, NTS = NT && RG_OPT_NT_STORE;
@@ -143,7 +146,7 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
     const float g = load1<G>(gp + (size_t)i * GS);
     float s1 = use_s1 ? *reinterpret_cast<const float*>(s1p + (size_t)i * 4) : 0.0f;
     float s2 = ALGO == kAdam ? *reinterpret_cast<const float*>(s2p + (size_t)i * 4) : 0.0f;
-    update_one<ALGO>(p, g, s1, s2, c, gscale);
+    update_one<ALGO>(p, g, s1, s2, c, coef);
     *reinterpret_cast<float*>(pp + (size_t)i * 4) = p;
     if (use_s1) *reinterpret_cast<float*>(s1p + (size_t)i * 4) = s1;
     if (ALGO == kAdam) *reinterpret_cast<float*>(s2p + (size_t)i * 4) = s2;
@@ -165,7 +168,7 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
     Codec<RG_F32, E>::unpack(r1, s1);
     Codec<RG_F32, E>::unpack(r2, s2);
 #pragma unroll
-    for (int j = 0; j < E; ++j) update_one<ALGO>(p[j], g[j], s1[j], s2[j], c, gscale);
+    for (int j = 0; j < E; ++j) update_one<ALGO>(p[j], g[j], s1[j], s2[j], c, coef);
     Mem<RG_F32, E, NTS>::store(pp + (size_t)e * 4, Codec<RG_F32, E>::pack(p));
     if (use_s1) Mem<RG_F32, E, NTS>::store(s1p + (size_t)e * 4, Codec<RG_F32, E>::pack(s1));
     if (ALGO == kAdam) Mem<RG_F32, E, NTS>::store(s2p + (size_t)e * 4, Codec<RG_F32, E>::pack(s2));
@@ -192,10 +195,10 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
 
 template <int ALGO, bool NT>
 __global__ __launch_bounds__(kOptThreads) void optim_kernel(OptArgs a) {
-  float gscale = a.c.grad_scale;
+  float coef = 1.0f;
   if (a.gate != nullptr) {
     if (a.gate->skipped != 0) return;
-    gscale = gscale * a.gate->coef;
+    coef = a.gate->coef;
   }
   const unsigned bid = blockIdx.x;
   const OptChunkRec r = a.chunks[bid / (unsigned)a.tiles_per_chunk];
@@ -210,7 +213,7 @@ __global__ __launch_bounds__(kOptThreads) void optim_kernel(OptArgs a) {
   const int copy_kind = r.copy ? r.copy_dtype : -1;
 #define RG_OPT(G, C)                                                       \
   if (r.grad_dtype == G && copy_kind == C) {                               \
-    optim_tile<ALGO, G, C, NT>(r, start, len, a.c, gscale);                \
+    optim_tile<ALGO, G, C, NT>(r, start, len, a.c, coef);                \
     return;                                                                \
   }
   RG_OPT(RG_F32, -1)

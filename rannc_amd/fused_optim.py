@@ -30,6 +30,20 @@ class _FusedBase(torch.optim.Optimizer):
         self.gate: int = 0
         #: every gradient is multiplied by this first
         self.grad_scale: float = 1.0
+        self._grad_sources: Dict[int, torch.Tensor] = {}
+
+    #: the step can read gradients from tensors other than ``param.grad`` (see ``set_grad_sources``)
+    reads_grad_sources = True
+
+    def set_grad_sources(self, params, grads) -> None:
+        """For the next steps ``grads[i]`` (any supported dtype, e.g. the still-scaled fp16 model
+        gradient) is read as the gradient of ``params[i]`` instead of ``params[i].grad``; together
+        with ``grad_scale`` and ``gate`` this folds unscale and clip into the step.  Empty lists
+        switch it off."""
+        self._grad_sources = {id(p): g for p, g in zip(params, grads) if g is not None}
+
+    def _grad_of(self, p: torch.Tensor) -> Optional[torch.Tensor]:
+        return self._grad_sources.get(id(p), p.grad) if self._grad_sources else p.grad
 
     # -- model copies (amp): written by the step kernel instead of a separate copy pass
     writes_model_copies = True
@@ -43,21 +57,22 @@ class _FusedBase(torch.optim.Optimizer):
             self._model_copies[id(m)] = c
         self._tables.clear()
 
-    def _check_param(self, p: torch.Tensor) -> None:
+    def _check_param(self, p: torch.Tensor, g: torch.Tensor) -> None:
         if p.dtype != torch.float32:
             raise ValueError(f"fused optimizers step fp32 parameters (masters), got {p.dtype}")
         if not p.is_cuda or not p.is_contiguous():
             raise ValueError("fused optimizers need contiguous GPU parameters")
-        if p.grad.is_sparse:
+        if g.is_sparse:
             raise ValueError("sparse gradients are not supported")
-        if not p.grad.is_contiguous() or p.grad.device != p.device or p.grad.numel() != p.numel():
+        if not g.is_contiguous() or g.device != p.device or g.numel() != p.numel():
             raise ValueError("gradient must be contiguous, on the parameter's device and of its size")
 
-    def _table(self, key: Tuple, params: List[torch.Tensor], state1: Optional[List[torch.Tensor]],
-               state2: Optional[List[torch.Tensor]]) -> _lib.OptimTable:
-        """Table for this exact list of parameters, re-pointed when any address moved."""
+    def _table(self, key: Tuple, params: List[torch.Tensor], grads: List[torch.Tensor],
+               state1: Optional[List[torch.Tensor]], state2: Optional[List[torch.Tensor]]) -> _lib.OptimTable:
+        """Table for this exact list of parameters and gradient dtypes, re-pointed when any address moved."""
         copies = [self._model_copies.get(id(p)) for p in params]
-        ptrs = (tuple(p.data_ptr() for p in params), tuple(p.grad.data_ptr() for p in params),
+        key = key + (tuple(g.dtype for g in grads),)
+        ptrs = (tuple(p.data_ptr() for p in params), tuple(g.data_ptr() for g in grads),
                 tuple(s.data_ptr() for s in state1) if state1 is not None else None,
                 tuple(s.data_ptr() for s in state2) if state2 is not None else None,
                 tuple(c.data_ptr() if c is not None else 0 for c in copies))
@@ -66,7 +81,7 @@ class _FusedBase(torch.optim.Optimizer):
         if hit is None:
             table = _lib.OptimTable(dev.index, ptrs[0], ptrs[1], ptrs[2], ptrs[3],
                                     ptrs[4] if any(ptrs[4]) else None, [p.numel() for p in params],
-                                    [dtype_code(p.grad.dtype) for p in params],
+                                    [dtype_code(g.dtype) for g in grads],
                                     [dtype_code(c.dtype) if c is not None else _lib.RG_F32 for c in copies])
         else:
             table, old, _ = hit
@@ -74,7 +89,7 @@ class _FusedBase(torch.optim.Optimizer):
                 table.update_pointers(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[4] if any(ptrs[4]) else None,
                                       stream_handle(dev))
         # the table borrows raw pointers: keep what it points at alive
-        self._tables[key] = (table, ptrs, [params, [p.grad for p in params], state1, state2, copies])
+        self._tables[key] = (table, ptrs, [params, grads, state1, state2, copies])
         return table
 
 
@@ -97,10 +112,13 @@ class FusedAdam(_FusedBase):
         for gi, group in enumerate(self.param_groups):
             by_step: Dict[int, List[torch.Tensor]] = {}
             step_tensors = []
+            grad_of: Dict[int, torch.Tensor] = {}
             for p in group["params"]:
-                if p.grad is None:
+                g = self._grad_of(p)
+                if g is None:
                     continue
-                self._check_param(p)
+                self._check_param(p, g)
+                grad_of[id(p)] = g
                 st = self.state[p]
                 if len(st) == 0:
                     st["step"] = torch.tensor(0.0, dtype=torch.float32)
@@ -119,7 +137,7 @@ class FusedAdam(_FusedBase):
             for step, ps in by_step.items():
                 ms = [self.state[p]["exp_avg"] for p in ps]
                 vs = [self.state[p]["exp_avg_sq"] for p in ps]
-                table = self._table((gi, tuple(id(p) for p in ps)), ps, ms, vs)
+                table = self._table((gi, tuple(id(p) for p in ps)), ps, [grad_of[id(p)] for p in ps], ms, vs)
                 b1, b2 = group["betas"]
                 table.adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], step,
                                 decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
@@ -156,10 +174,13 @@ class FusedSGD(_FusedBase):
                 loss = closure()
         for gi, group in enumerate(self.param_groups):
             fresh, seasoned = [], []
+            grad_of: Dict[int, torch.Tensor] = {}
             for p in group["params"]:
-                if p.grad is None:
+                g = self._grad_of(p)
+                if g is None:
                     continue
-                self._check_param(p)
+                self._check_param(p, g)
+                grad_of[id(p)] = g
                 st = self.state[p]
                 if group["momentum"] != 0 and st.get("momentum_buffer") is None:
                     st["momentum_buffer"] = torch.empty_like(p, memory_format=torch.preserve_format)
@@ -170,7 +191,7 @@ class FusedSGD(_FusedBase):
                 if not ps:
                     continue
                 bufs = [self.state[p]["momentum_buffer"] for p in ps] if group["momentum"] != 0 else None
-                table = self._table((gi, first, tuple(id(p) for p in ps)), ps, bufs, None)
+                table = self._table((gi, first, tuple(id(p) for p in ps)), ps, [grad_of[id(p)] for p in ps], bufs, None)
                 table.sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
                                group["nesterov"], group["maximize"], first_step=first, grad_scale=self.grad_scale,
                                gate=self.gate, stream=stream_handle(ps[0].device))

@@ -128,6 +128,9 @@ class TensorPlan:
     def step_finish(self, max_norm: float, flags: int = _lib.RG_STEP_DEFAULT) -> None:
         self.plan.step_finish(max_norm, flags, self._stream())
 
+    def step_decide(self, max_norm: float, flags: int = _lib.RG_STEP_DEFAULT) -> None:
+        self.plan.step_decide(max_norm, flags, self._stream())
+
     def unscale_pack(self, inv_scale: float) -> None:
         self.plan.unscale_pack(inv_scale, self._stream())
 

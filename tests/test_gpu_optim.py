@@ -230,44 +230,93 @@ def test_bad_arguments_are_value_errors():
 
 
 def test_whole_step_fused_unscale_clip_then_fused_adam():
-    """scale_loss (read pass) -> clip_grad_norm (write pass, clipped) -> FusedAdam.step (masters +
-    model copies), against the oracle's sequence unscale -> norm -> clip -> Adam -> half(master)."""
-    torch.manual_seed(11)
+    """scale_loss (read pass) -> clip_grad_norm -> FusedAdam.step, two ways: (A) the clipped master
+    gradients are written (write pass) and Adam reads them; (B) nothing is written, the step kernel
+    reads the scaled model gradients and the clip decision from the device.  A is checked against
+    the oracle's sequence unscale -> norm -> clip -> Adam -> half(master); B must equal A bit for bit."""
+    import copy
     half = torch.bfloat16
-    model = torch.nn.Sequential(torch.nn.Linear(64, 96), torch.nn.Tanh(), torch.nn.Linear(96, 10)).to(DEV)
-    opt = FusedAdam(model.parameters(), lr=5e-3, weight_decay=0.01)
-    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 10, half_dtype=half, fused=True)
-    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    torch.manual_seed(11)
+    base = torch.nn.Sequential(torch.nn.Linear(64, 96), torch.nn.Tanh(), torch.nn.Linear(96, 10)).to(DEV)
+    flows = {}
+    for name in ("A", "B"):
+        model = copy.deepcopy(base)
+        opt = FusedAdam(model.parameters(), lr=5e-3, weight_decay=0.01)
+        model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 10, half_dtype=half, fused=True)
+        flows[name] = (model, opt, rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True))
     ms = vs = None
+    g = torch.Generator().manual_seed(12)
     for it in range(3):
-        x = torch.randn(32, 64, device=DEV, dtype=half)
-        loss = rm(x).float().pow(2).sum()
-        with amp.scale_loss(loss, opt) as scaled:
-            scaled.backward()
-            model_grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
-        stash = opt._amp_stash
-        masters = stash.all_fp32_from_fp16_params
-        scale = 2.0 ** 10
-        rm.clip_grad_norm(0.5)
-        want = oracle.fused_step(model_grads, ["f32"] * len(model_grads), 1.0 / scale, 0.5)
-        assert want.coef is not None, "the test is meant to clip"
-        offs = 0
-        want_grads = []
-        for m in masters:
-            want_grads.append(want.buckets["f32"][offs:offs + m.numel()].view(m.shape))
-            offs += m.numel()
-        for m, w in zip(masters, want_grads):
-            torch.testing.assert_close(m.grad.cpu(), w, rtol=2e-6, atol=0.0)      # coef agrees to 1e-6, values follow
-        m_cpu = [m.detach().cpu().clone() for m in masters]
-        g_cpu = [m.grad.detach().cpu().clone() for m in masters]
-        if ms is None:
-            ms = [torch.zeros_like(t) for t in m_cpu]
-            vs = [torch.zeros_like(t) for t in m_cpu]
-        opt.step()
-        oracle_optim.adam_step(m_cpu, g_cpu, ms, vs, it + 1, lr=5e-3, weight_decay=0.01)
-        for m, w, p in zip(masters, m_cpu, stash.all_fp16_params):
-            close(m, w, 5e-3 * RTOL, f"master it {it}")
-            assert_bits_equal(p.detach().cpu(), oracle_optim.model_copy(m.detach().cpu(), half), "model copy")
-        for a, b, m in zip(ms, vs, masters):
-            a.copy_(opt.state[m]["exp_avg"]); b.copy_(opt.state[m]["exp_avg_sq"])
-        opt.zero_grad()          # master gradients go back to None: the next unscale overwrites (else it accumulates)
+        x = torch.randn(32, 64, generator=g).to(DEV).to(half)
+        results = {}
+        for name, (model, opt, rm) in flows.items():
+            loss = rm(x).float().pow(2).sum()
+            with amp.scale_loss(loss, opt) as scaled:
+                scaled.backward()
+                model_grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
+            stash = opt._amp_stash
+            masters = stash.all_fp32_from_fp16_params
+            rm.clip_grad_norm(0.5)
+            assert stash.pending_finish and stash.decided_max_norm == 0.5          # only the decision was taken
+            if name == "A":
+                amp.finish_unscale(opt)                                             # write the clipped master gradients
+                want = oracle.fused_step(model_grads, ["f32"] * len(model_grads), 1.0 / 2.0 ** 10, 0.5)
+                assert want.coef is not None, "the test is meant to clip"
+                offs = 0
+                for m in masters:
+                    w = want.buckets["f32"][offs:offs + m.numel()].view(m.shape)
+                    torch.testing.assert_close(m.grad.cpu(), w, rtol=2e-6, atol=0.0)  # coef agrees to 1e-6, values follow
+                    offs += m.numel()
+                m_cpu = [m.detach().cpu().clone() for m in masters]
+                g_cpu = [m.grad.detach().cpu().clone() for m in masters]
+                if ms is None:
+                    ms = [torch.zeros_like(t) for t in m_cpu]
+                    vs = [torch.zeros_like(t) for t in m_cpu]
+            opt.step()
+            assert not stash.pending_finish
+            if name == "A":
+                oracle_optim.adam_step(m_cpu, g_cpu, ms, vs, it + 1, lr=5e-3, weight_decay=0.01)
+                for m, w, p in zip(masters, m_cpu, stash.all_fp16_params):
+                    close(m, w, 5e-3 * RTOL, f"master it {it}")
+                    assert_bits_equal(p.detach().cpu(), oracle_optim.model_copy(m.detach().cpu(), half), "model copy")
+                for a, b, m in zip(ms, vs, masters):
+                    a.copy_(opt.state[m]["exp_avg"]); b.copy_(opt.state[m]["exp_avg_sq"])
+            results[name] = ([m.detach().cpu().clone() for m in masters],
+                             [p.detach().cpu().clone() for p in stash.all_fp16_params],
+                             [opt.state[m]["exp_avg_sq"].cpu().clone() for m in masters])
+            opt.zero_grad()          # master gradients go back to None: the next unscale overwrites (else it accumulates)
+        for k in range(3):
+            for a, b in zip(results["A"][k], results["B"][k]):
+                assert_bits_equal(b, a, f"direct step vs materialised step, it {it}")
+
+
+def test_direct_step_skips_on_overflow_and_without_clip_call():
+    half = torch.float16
+    torch.manual_seed(13)
+    model = torch.nn.Sequential(torch.nn.Linear(16, 16), torch.nn.Linear(16, 4)).to(DEV)
+    opt = FusedSGD(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, half_dtype=half, fused=True)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    x = torch.randn(8, 16, device=DEV, dtype=half)
+    # no clip_grad_norm at all: the step takes the (no-clip) decision itself
+    loss = rm(x).float().pow(2).mean()
+    with amp.scale_loss(loss, opt) as scaled:
+        scaled.backward()
+        grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
+    masters = opt._amp_stash.all_fp32_from_fp16_params
+    before = [m.detach().cpu().clone() for m in masters]
+    opt.step()
+    unscaled, _ = oracle.unscale_and_check(grads, 1.0 / 256.0)
+    oracle_optim.sgd_step(before, unscaled, None, 0.1)
+    for m, w in zip(masters, before):
+        close(m, w, 1e-8, "sgd from model grads")
+    opt.zero_grad()
+    # overflow: the scaler arms the skip; nothing may change
+    loss = rm(x).float().pow(2).mean() * float("inf")
+    with amp.scale_loss(loss, opt) as scaled:
+        scaled.backward()
+    snap = [m.detach().clone() for m in masters]
+    opt.step()
+    for m, s0 in zip(masters, snap):
+        assert torch.equal(m, s0)
+    assert amp._amp_state.loss_scalers[0].loss_scale() == 128.0
