@@ -126,6 +126,12 @@ class Plan {
   void fused_step(float inv_scale, float max_norm, int flags) { check(rg_fused_step(handle(), inv_scale, max_norm, flags, current_stream(device_))); }
   void step_begin(float inv_scale) { check(rg_step_begin(handle(), inv_scale, current_stream(device_))); }
   void step_finish(float max_norm, int flags) { check(rg_step_finish(handle(), max_norm, flags, current_stream(device_))); }
+  void step_decide(float max_norm, int flags) { check(rg_step_decide(handle(), max_norm, flags, current_stream(device_))); }
+  uintptr_t result_device_ptr() {
+    const rg_step_result* r = nullptr;
+    check(rg_result_device_ptr(handle(), &r));
+    return reinterpret_cast<uintptr_t>(r);
+  }
   void unscale_pack(float inv_scale) { check(rg_unscale_pack(handle(), inv_scale, current_stream(device_))); }
   void accumulate(float scale) { check(rg_accumulate(handle(), scale, current_stream(device_))); }
   void unscale_accumulate(float inv_scale) {
@@ -226,13 +232,15 @@ class Optim {
     }
   }
   void adam_step(double lr, double beta1, double beta2, double eps, double weight_decay, int64_t step, bool decoupled,
-                 bool maximize, float grad_scale) {
-    rg_adam_args a{lr, beta1, beta2, eps, weight_decay, step, decoupled ? 1 : 0, maximize ? 1 : 0, grad_scale, nullptr};
+                 bool maximize, float grad_scale, uintptr_t gate) {
+    rg_adam_args a{lr, beta1, beta2, eps, weight_decay, step, decoupled ? 1 : 0, maximize ? 1 : 0, grad_scale,
+                   reinterpret_cast<const rg_step_result*>(gate)};
     check(rg_adam_step(handle(), &a, current_stream(device_)));
   }
   void sgd_step(double lr, double momentum, double dampening, double weight_decay, bool nesterov, bool maximize,
-                bool first_step, float grad_scale) {
-    rg_sgd_args a{lr, momentum, dampening, weight_decay, nesterov ? 1 : 0, maximize ? 1 : 0, first_step ? 1 : 0, grad_scale, nullptr};
+                bool first_step, float grad_scale, uintptr_t gate) {
+    rg_sgd_args a{lr, momentum, dampening, weight_decay, nesterov ? 1 : 0, maximize ? 1 : 0, first_step ? 1 : 0, grad_scale,
+                  reinterpret_cast<const rg_step_result*>(gate)};
     check(rg_sgd_step(handle(), &a, current_stream(device_)));
   }
 
@@ -288,6 +296,8 @@ PYBIND11_MODULE(_ranncgrad, m) {
       .def("fused_step", &Plan::fused_step, py::arg("inv_scale"), py::arg("max_norm"), py::arg("flags") = 0)
       .def("step_begin", &Plan::step_begin)
       .def("step_finish", &Plan::step_finish, py::arg("max_norm"), py::arg("flags") = 0)
+      .def("step_decide", &Plan::step_decide, py::arg("max_norm"), py::arg("flags") = 0)
+      .def("result_device_ptr", &Plan::result_device_ptr)
       .def("unscale_pack", &Plan::unscale_pack)
       .def("accumulate", &Plan::accumulate, py::arg("scale") = 1.0f)
       .def("unscale_accumulate", &Plan::unscale_accumulate)
@@ -307,9 +317,9 @@ PYBIND11_MODULE(_ranncgrad, m) {
            py::arg("model_copies") = py::none())
       .def("adam_step", &Optim::adam_step, py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("eps"),
            py::arg("weight_decay"), py::arg("step"), py::arg("decoupled") = false, py::arg("maximize") = false,
-           py::arg("grad_scale") = 1.0f)
+           py::arg("grad_scale") = 1.0f, py::arg("gate") = (uintptr_t)0)
       .def("sgd_step", &Optim::sgd_step, py::arg("lr"), py::arg("momentum") = 0.0, py::arg("dampening") = 0.0,
            py::arg("weight_decay") = 0.0, py::arg("nesterov") = false, py::arg("maximize") = false,
-           py::arg("first_step") = false, py::arg("grad_scale") = 1.0f)
+           py::arg("first_step") = false, py::arg("grad_scale") = 1.0f, py::arg("gate") = (uintptr_t)0)
       .def("close", &Optim::close);
 }

@@ -95,6 +95,13 @@ def test_optimizer_table_through_pybind_matches_ctypes():
         ob.adam_step(1e-3, 0.9, 0.999, 1e-8, 0.01, step, stream=stream_handle(dev))
     oa.sgd_step(0.1)
     ob.sgd_step(0.1, stream=stream_handle(dev))
+    # the clip decision of a plan, consumed on the device by both bindings
+    pl = _ranncgrad.Plan(grads, [torch.zeros_like(t) for t in grads])
+    pl.step_begin(1.0)
+    pl.step_decide(1e-3)
+    assert pl.result()["clipped"] == 1
+    oa.sgd_step(0.1, gate=pl.result_device_ptr())
+    ob.sgd_step(0.1, gate=pl.result_device_ptr(), stream=stream_handle(dev))
     for k in "pmvc":
         for x, y in zip(a[k], b[k]):
             assert_bits_equal(x.cpu(), y.cpu(), f"pybind vs ctypes {k}")
