@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # HBM traffic per launch of the dominant kernel (the write pass), from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs of this same command, each scaled by what the counter reads for
 # a plain 1 GiB copy (profiles/fused_step_c2_bert_large_hbm_traffic.txt).  Missing = not measured.
-MEASURED_TRAFFIC_BYTES = {"c2_bert_large": 2021550504}
+MEASURED_TRAFFIC_BYTES = {"c2_bert_large": 2021548222}
 # the Adam step with bf16 model copy, same method (profiles/adam_step_c2_bert_large_kernel_stats.txt)
 MEASURED_TRAFFIC_BYTES_ADAM = {"c2_bert_large": 10075311450}
 
