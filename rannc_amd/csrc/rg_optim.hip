@@ -54,19 +54,26 @@ struct OptArgs {
   OptConst c;
 };
 
-#ifndef RG_OPT_THREADS
-#define RG_OPT_THREADS 128
+// Launch shape per algorithm, measured on MI355X over BERT-large's tensors: SGD (3-4 streams)
+// is fastest in the shape of the gradient path's writing passes; Adam (8 streams) gains 1-2 %
+// from larger blocks over larger tiles with four vectors per array in flight.
+template <int ALGO> struct OptShape;
+template <> struct OptShape<kAdam> {
+#if defined(RG_OPT_THREADS)
+  static constexpr int kThreads = RG_OPT_THREADS, kTileElems = RG_OPT_TILE_ELEMS, kUnroll = RG_OPT_UNROLL;
+#else
+  static constexpr int kThreads = 256, kTileElems = 4096, kUnroll = 4;
 #endif
-#ifndef RG_OPT_TILE_ELEMS
-#define RG_OPT_TILE_ELEMS 1024
+};
+template <> struct OptShape<kSgd> {
+#if defined(RG_OPT_THREADS)
+  static constexpr int kThreads = RG_OPT_THREADS, kTileElems = RG_OPT_TILE_ELEMS, kUnroll = RG_OPT_UNROLL;
+#else
+  static constexpr int kThreads = 128, kTileElems = 1024, kUnroll = 1;
 #endif
-#ifndef RG_OPT_UNROLL
-#define RG_OPT_UNROLL 1
-#endif
-constexpr int kOptThreads = RG_OPT_THREADS;
-constexpr int kOptTileElems = RG_OPT_TILE_ELEMS;
+};
+constexpr int kOptMinTileElems = 1024;   // smallest tile of any shape (bounds the grid size of a table)
 constexpr int kOptE = 4;    // elements per lane per instruction
-constexpr int kOptU = RG_OPT_UNROLL;   // vectors per array a lane has in flight
 #ifndef RG_OPT_NT_LOAD
 #define RG_OPT_NT_LOAD 1
 #endif
@@ -116,7 +123,7 @@ template <> __device__ __forceinline__ float load1<RG_BF16>(const char* p) {
 // One tile of one chunk.  G: gradient dtype; C: model-copy dtype, or -1 for none.
 template <int ALGO, int G, int C, bool NT>
 __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int len, const OptConst& c, float coef) {
-  constexpr int T = kOptThreads;
+  constexpr int T = OptShape<ALGO>::kThreads;
   constexpr int E = kOptE;
   constexpr bool NTL = NT && RG_OPT_NT_LOAD, NTS = NT && RG_OPT_NT_STORE;
   constexpr int GS = ElemSize<G>::value;
@@ -174,7 +181,7 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
     if (ALGO == kAdam) Mem<RG_F32, E, NTS>::store(s2p + (size_t)e * 4, Codec<RG_F32, E>::pack(s2));
     if constexpr (kCopy) Mem<CD, E, NTS>::store(cp + (size_t)e * CS, Codec<CD, E>::pack(p));
   };
-  constexpr int U = kOptU;
+  constexpr int U = OptShape<ALGO>::kUnroll;
   constexpr int kIter = T * E * U;
   int base = head;
   for (; base + kIter <= tail0; base += kIter) {     // all loads of U steps in flight together
@@ -194,7 +201,7 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
 }
 
 template <int ALGO, bool NT>
-__global__ __launch_bounds__(kOptThreads) void optim_kernel(OptArgs a) {
+__global__ __launch_bounds__(OptShape<ALGO>::kThreads) void optim_kernel(OptArgs a) {
   float coef = 1.0f;
   if (a.gate != nullptr) {
     if (a.gate->skipped != 0) return;
@@ -346,7 +353,7 @@ RG_API int rg_optim_create(rg_optim** out, int device, int n, void* const* param
   }
   o->n_chunks = o->chunk_begin[(size_t)n];
   int rc = check_rows(o, "rg_optim_create");
-  const int64_t tiles = (o->chunk_elems + kOptTileElems - 1) / kOptTileElems;
+  const int64_t tiles = (o->chunk_elems + kOptMinTileElems - 1) / kOptMinTileElems;
   if (rc == RG_OK && o->n_chunks * tiles > 0x7fffffffLL) {
     set_error("rg_optim_create: %lld elements exceed one launch", (long long)o->total_numel);
     rc = RG_EINVAL;
@@ -439,10 +446,10 @@ static int launch_optim(const rg_optim* o, const OptConst& c, const rg_step_resu
   memset(&a, 0, sizeof(a));
   a.chunks = o->d_chunks;
   a.gate = reinterpret_cast<const StepResult*>(gate);
-  a.tile_elems = kOptTileElems;
-  a.tiles_per_chunk = (int32_t)((o->chunk_elems + kOptTileElems - 1) / kOptTileElems);
+  a.tile_elems = OptShape<ALGO>::kTileElems;
+  a.tiles_per_chunk = (int32_t)((o->chunk_elems + OptShape<ALGO>::kTileElems - 1) / OptShape<ALGO>::kTileElems);
   a.c = c;
-  const dim3 grid((unsigned)(o->n_chunks * a.tiles_per_chunk)), block(kOptThreads);
+  const dim3 grid((unsigned)(o->n_chunks * a.tiles_per_chunk)), block(OptShape<ALGO>::kThreads);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (o->total_numel * bytes_per_elem > ((int64_t)256 << 20)) hipLaunchKernelGGL((optim_kernel<ALGO, true>), grid, block, 0, s, a);
   else hipLaunchKernelGGL((optim_kernel<ALGO, false>), grid, block, 0, s, a);
