@@ -293,10 +293,12 @@ def test_amp_step_matches_oracle_sequence(fused, half):
     rm.zero_grad()
 
 
-def test_amp_gradient_accumulation_adds_into_live_master_grads():
+@pytest.mark.parametrize("fused,fused_opt", [(False, False), (True, False), (True, True)])
+def test_amp_gradient_accumulation_adds_into_live_master_grads(fused, fused_opt):
+    from rannc_amd.fused_optim import FusedSGD
     model = _tiny_model()
-    opt = torch.optim.SGD(model.parameters(), lr=0.1)
-    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8)
+    opt = (FusedSGD if fused_opt else torch.optim.SGD)(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, fused=fused)
     rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
     xs = [torch.randn(16, 32, device=DEV, dtype=torch.float16) for _ in range(3)]
     want = None
