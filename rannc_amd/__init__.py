@@ -101,7 +101,41 @@ class RaNNCModule(_pyrannc.RaNNCModule):
         if self.enable_zero:
             self.sync_param_zero(False)                               # GraphLauncher.cpp:366-368
         self.prepare_backward()                                       # GraphLauncher.cpp:468
-        return self.model(*args, **kwargs)
+        out = self.model(*args, **kwargs)
+        if torch.is_grad_enabled():
+            self._hook_end_of_backward(out)
+        return out
+
+    def _hook_end_of_backward(self, out) -> None:
+        """What the reference does when a backward pass through the module ends
+        (``GraphLauncher::backward``, ``src/comp/GraphLauncher.cpp:484-486``, then
+        ``RaNNCTensorBackward::apply``, ``src/comp/Backward.cpp:101-108``): point the gradients of
+        the ZeRO segments at their slice of the parameters' gradients and run the gradient
+        exchange (for one process: the staging pack and copy-back).  Hooked on the outputs and
+        run once, after autograd has produced every gradient of the pass."""
+        tensors = [t for t in (out if isinstance(out, (tuple, list)) else [out])
+                   if isinstance(t, torch.Tensor) and t.requires_grad]
+        if not tensors:
+            return
+        state = {"queued": False}
+
+        def at_end():
+            state["queued"] = False
+            with torch.no_grad():
+                if self.enable_zero:
+                    self.set_grad_to_local_param_segment()
+                    self.allreduce_grads_zero()
+                else:
+                    self.allreduce_grads()
+
+        def on_grad(grad):
+            if not state["queued"]:
+                state["queued"] = True
+                torch.autograd.Variable._execution_engine.queue_callback(at_end)
+            return grad
+
+        for t in tensors:
+            t.register_hook(on_grad)
 
     def parameters(self, *args, **kwargs):
         return self.model.parameters(*args, **kwargs)

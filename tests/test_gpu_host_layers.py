@@ -457,3 +457,36 @@ def test_amp_accumulates_fp32_parameter_gradients_too():
             oracle.unscale_accumulate(want_w, [scaled_grad], 1.0 / 256.0)
         assert_bits_equal(model[1].weight.grad.cpu(), want_w[0], f"bn weight grad after {it + 1} micro-batches")
     opt.step()
+
+
+@pytest.mark.parametrize("fused,fused_opt", [(False, False), (True, False), (True, True)])
+def test_zero_mode_trains_exactly_like_the_plain_mode(fused, fused_opt):
+    """The reference's own invariant for ZeRO (test/common.py compares the partitioned run with the
+    plain one): with one process the segments are the whole parameters, so three training steps with
+    ``enable_zero`` must leave bit-identical masters and model parameters."""
+    import copy
+    from rannc_amd.fused_optim import FusedAdam
+    torch.manual_seed(21)
+    base = torch.nn.Sequential(torch.nn.Linear(32, 50), torch.nn.Tanh(), torch.nn.Linear(50, 9)).to(DEV)   # odd sizes: padded segments
+    g = torch.Generator().manual_seed(22)
+    xs = [torch.randn(16, 32, generator=g).to(DEV).half() for _ in range(3)]
+    finals = {}
+    for zero in (False, True):
+        _pyrannc.clear()
+        model = copy.deepcopy(base)
+        opt = FusedAdam(model.parameters(), lr=1e-2) if fused_opt else torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9)
+        model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, fused=fused)
+        rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True, enable_zero=zero)
+        for x in xs:
+            loss = rm(x).float().pow(2).mean()
+            with amp.scale_loss(loss, opt) as scaled:
+                scaled.backward()
+            rm.clip_grad_norm(0.05)
+            opt.step()
+            opt.zero_grad()
+        finals[zero] = ([p.detach().cpu().clone().flatten() for p in model.parameters()],
+                        [m.detach().cpu().clone().flatten() for m in opt._amp_stash.all_fp32_from_fp16_params])
+        assert not torch.equal(finals[zero][0][0], base[0].weight.detach().cpu().half().flatten()), "the step did nothing"
+    for k in (0, 1):
+        for a, b in zip(finals[False][k], finals[True][k]):
+            assert_bits_equal(b[:a.numel()], a, "zero vs plain")
