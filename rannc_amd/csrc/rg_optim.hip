@@ -95,13 +95,8 @@ __device__ __forceinline__ void update_one(float& p, float g, float& s1, float& 
     s1 = __builtin_fmaf(c.lerp_coeff, g - s1, c.lerp_from_end ? g : s1);
     // exp_avg_sq.mul_(beta2).addcmul_(g, g, value = 1 - beta2)
     s2 = __builtin_fmaf(c.one_minus_beta2 * g, g, s2 * c.beta2);
-#ifdef RG_ADAM_FAST_MATH   // diagnostic build only: approximate sqrt / reciprocal
-    const float denom = __builtin_amdgcn_sqrtf(s2) * c.bias2_sqrt + c.eps;
-    p = p + (c.neg_step_size * s1) * __builtin_amdgcn_rcpf(denom);
-#else
-    const float denom = sqrtf(s2) / c.bias2_sqrt + c.eps;
+    const float denom = sqrtf(s2) / c.bias2_sqrt + c.eps;          // correctly rounded sqrt and divisions
     p = p + (c.neg_step_size * s1) / denom;
-#endif
   } else {
     if (c.weight_decay != 0.0f) g = __builtin_fmaf(c.weight_decay, p, g);
     if (c.has_momentum) {
