@@ -400,6 +400,10 @@ RG_API int rg_optim_update_pointers(rg_optim* o, void* const* param, const void*
     set_error("rg_optim_update_pointers: null table");
     return RG_EINVAL;
   }
+  if ((state1 != nullptr && !o->has_state1) || (state2 != nullptr && !o->has_state2)) {
+    set_error("rg_optim_update_pointers: the table was created without these state arrays");
+    return RG_EINVAL;
+  }
   std::vector<rg_optim::Row> saved = o->rows;
   for (int i = 0; i < o->n_tensors; ++i) {
     rg_optim::Row& t = o->rows[(size_t)i];
