@@ -271,8 +271,12 @@ int rg_sgd_step(rg_optim* opt, const rg_sgd_args* args, void* stream);
  * returns milliseconds: ms[0] reduce pass, ms[1] finalize, ms[2] write pass, ms[3] whole step.
  * slot counts fused steps since timing was enabled, modulo `slots`.
  * A negative `slots` brackets only the write pass (two records per step instead of four, for
- * measurements where the records' own cost matters); ms[0], ms[1], ms[3] then read -1. */
+ * measurements where the records' own cost matters); ms[0], ms[1], ms[3] then read -1.
+ * rg_plan_timing_stride(plan, k) brackets only every k-th step (slot = bracketed steps modulo
+ * `slots`): each event record costs a few microseconds of stream time, so sampling keeps a
+ * measurement loop close to the untimed one. */
 int rg_plan_enable_timing(rg_plan* plan, int slots);
+int rg_plan_timing_stride(rg_plan* plan, int stride);
 int rg_plan_read_timing(rg_plan* plan, int slot, float ms[4]);
 
 #ifdef __cplusplus

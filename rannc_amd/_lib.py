@@ -77,6 +77,7 @@ SIGNATURES = {
     "rg_adam_step": (_i, [_vp, C.POINTER(AdamArgs), _vp]),
     "rg_sgd_step": (_i, [_vp, C.POINTER(SgdArgs), _vp]),
     "rg_plan_enable_timing": (_i, [_vp, _i]),
+    "rg_plan_timing_stride": (_i, [_vp, _i]),
     "rg_plan_read_timing": (_i, [_vp, _i, C.POINTER(C.c_float)]),
 }
 
@@ -245,6 +246,9 @@ class Plan:
     def enable_timing(self, slots: int) -> None:
         """slots > 0: bracket all stages of each fused step; < 0: only the write pass; 0: off."""
         check(lib.rg_plan_enable_timing(self._handle, slots))
+
+    def timing_stride(self, stride: int) -> None:
+        check(lib.rg_plan_timing_stride(self._handle, stride))
 
     def read_timing(self, slot: int) -> List[float]:
         """[reduce pass, finalize, write pass, whole step] in milliseconds."""

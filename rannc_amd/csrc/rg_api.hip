@@ -73,7 +73,9 @@ struct rg_plan {
   // optional ring of event quadruples around the kernels of rg_fused_step
   std::vector<hipEvent_t> timing_events;
   int timing_slots = 0;
-  int64_t timing_count = 0;
+  int64_t timing_count = 0;   // steps bracketed so far
+  int64_t timing_steps = 0;   // steps seen so far
+  int timing_stride = 1;      // every stride-th step is bracketed
   bool timing_all = true;  // false: only the write pass is bracketed (two records per step)
 };
 
@@ -483,7 +485,8 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   hipEvent_t* ev = nullptr;
-  if (p->timing_slots > 0) ev = &p->timing_events[(size_t)(p->timing_count++ % p->timing_slots) * 4];
+  if (p->timing_slots > 0 && p->timing_steps++ % p->timing_stride == 0)
+    ev = &p->timing_events[(size_t)(p->timing_count++ % p->timing_slots) * 4];
   PassArgs a = pass_args(p, inv_scale);
   const bool all = ev != nullptr && p->timing_all;
   if (all) RG_HIP(hipEventRecord(ev[0], s));
@@ -754,6 +757,7 @@ RG_API int rg_plan_enable_timing(rg_plan* p, int slots) {
   p->timing_events.clear();
   p->timing_slots = 0;
   p->timing_count = 0;
+  p->timing_steps = 0;
   p->timing_events.reserve((size_t)slots * 4);
   for (int i = 0; i < slots * 4; ++i) {
     hipEvent_t e;
@@ -761,6 +765,16 @@ RG_API int rg_plan_enable_timing(rg_plan* p, int slots) {
     p->timing_events.push_back(e);
   }
   p->timing_slots = slots;
+  return RG_OK;
+}
+
+RG_API int rg_plan_timing_stride(rg_plan* p, int stride) {
+  if (p == nullptr || stride < 1) {
+    set_error("rg_plan_timing_stride: bad arguments");
+    return RG_EINVAL;
+  }
+  p->timing_stride = stride;
+  p->timing_steps = 0;
   return RG_OK;
 }
 
