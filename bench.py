@@ -31,8 +31,8 @@ MEASURED_TRAFFIC_BYTES_ADAM = {"c2_bert_large": 10075311450}
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_bert_large")
     ap.add_argument("--op", default="fused_step", choices=["fused_step", "adam", "sgd", "adam_from_model_grads"],
                     help="fused_step (default: the graded metric), the optimizer step that follows it, or both "
