@@ -202,3 +202,37 @@ def test_repeatable_bits():
     b = _run_fused(grads, torch.float32, 1 / 1024.0, 0.1)
     assert a[0].norm == b[0].norm and a[0].coef == b[0].coef and a[1] == b[1]
     assert_bits_equal(a[2], b[2], "run-to-run")
+
+
+@pytest.mark.parametrize("env", [
+    {"RG_XCD_REDUCE": "-1"}, {"RG_XCD_REDUCE": "3", "RG_XCD_WRITE": "5"}, {"RG_XCD_WRITE": "-1"},
+    {"RG_WRITE_TILE_ELEMS": "256"}, {"RG_WRITE_TILE_ELEMS": "4096", "RG_REDUCE_TILE_FACTOR": "4"},
+    {"RG_REDUCE_TILE_FACTOR": "1"},
+])
+def test_tuning_knobs_do_not_change_results(env, monkeypatch):
+    """Block -> XCD mappings and tile sizes only reorder the work: values are bit-identical, sums
+    within the norm tolerance (their order changes with the tile size)."""
+    g = torch.Generator().manual_seed(77)
+    cpu = [(torch.randn(n, generator=g) * 8).to(torch.bfloat16) for n in (100003, 5, 16384, 40000, 1, 262147)]
+    srcs = [t.to("cuda:0") for t in cpu]
+    ref_out = [torch.zeros(t.shape, device="cuda:0") for t in cpu]
+    ref = TensorPlan(srcs, ref_out, chunk_elems=4096)
+    ref.fused_step(0.125, 0.5)
+    want = ref.result()
+    ref_pack = [torch.zeros(t.shape, device="cuda:0") for t in cpu]
+    rp = TensorPlan(srcs, ref_pack, chunk_elems=4096)
+    rp.unscale_pack(0.125)
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    out = [torch.full(t.shape, 3.0, device="cuda:0") for t in cpu]
+    plan = TensorPlan(srcs, out, chunk_elems=4096)           # the knobs are read when the plan is created
+    plan.fused_step(0.125, 0.5)
+    got = plan.result()
+    assert (got.overflow, got.clipped) == (want.overflow, want.clipped) and got.clipped == 1
+    assert got.norm == want.norm and got.coef == want.coef       # the read pass keeps its chunk partials whatever the mapping
+    for a, b in zip(out, ref_out):
+        assert_bits_equal(a.cpu(), b.cpu(), f"fused step with {env}")
+    plan.unscale_pack(0.125)
+    assert math.isclose(plan.result().norm, rp.result().norm, rel_tol=1e-12)
+    for a, b in zip(out, ref_pack):
+        assert_bits_equal(a.cpu(), b.cpu(), f"unscale_pack with {env}")
