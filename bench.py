@@ -152,7 +152,7 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
         else:
             table.sgd_step(0.01, stream=st)
 
-    for _ in range(args.warmup):
+    for _ in range(max(0, 20 - args.warmup) + args.warmup):      # warm-up, at least 20 steps so the clocks have ramped
         step()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -161,6 +161,8 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
     for _ in range(args.steps):
         step()
     e1.record()
+    while not e1.query():             # poll: a blocking wait adds its wake-up latency to the last step
+        pass
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     launch_ms = e0.elapsed_time(e1) / args.steps
@@ -274,13 +276,15 @@ def main() -> int:
     s, d = grads[0].element_size(), bucket.element_size()
 
     plan = TensorPlan(grads, dsts, chunk_elems=args.chunk_elems)
-    for _ in range(args.warmup):
+    # Untimed: the W warm-up steps asked for, preceded by enough further steps (about 25 ms of work)
+    # that the GPU has left its idle clocks before anything is timed.
+    for _ in range(max(0, 60 - args.warmup) + args.warmup):
         plan.fused_step(cfg.inv_scale, cfg.max_norm)
     torch.cuda.synchronize()
     # Timed region: HIP events (recorded by the library on the launch stream) bracket only the
     # dominant kernel, the write pass, and only on every fifth step: each record costs a few
     # microseconds of stream time, which would otherwise be part of every step measured here.
-    stride = 5 if args.steps >= 10 else 1
+    stride = min(5, max(1, args.steps))
     sampled = (args.steps + stride - 1) // stride
     plan.plan.enable_timing(-sampled)
     plan.plan.timing_stride(stride)
@@ -288,6 +292,10 @@ def main() -> int:
     t0 = time.perf_counter()
     for _ in range(args.steps):
         plan.fused_step(cfg.inv_scale, cfg.max_norm)
+    done = torch.cuda.Event()
+    done.record()
+    while not done.query():       # poll: a blocking wait adds its wake-up latency to the last step
+        pass
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     res = plan.result()
@@ -336,7 +344,8 @@ def main() -> int:
                    "src_bytes_per_elem": s, "dst_bytes_per_elem": d,
                    "algorithmic_bytes_per_step": step_bytes, "clipped": clipped, "overflow": int(res.overflow),
                    "norm": res.norm, "coef": res.coef, "seed": args.seed,
-                   "chunk_elems": plan.plan.chunk_elems, "chunks": plan.plan.num_chunks},
+                   "chunk_elems": plan.plan.chunk_elems, "chunks": plan.plan.num_chunks,
+                   "untimed_steps_before_timing": max(0, 60 - args.warmup) + args.warmup},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "elements_per_s": round(n / step_s, 1),
         "roofline": roofline,
