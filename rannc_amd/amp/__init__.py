@@ -310,7 +310,14 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
         if p.grad is not None:
             stashed_fp32[id(p)] = p.grad
             p.grad = None
-    yield loss.float() * scaler.loss_scale()
+    try:
+        yield loss.float() * scaler.loss_scale()
+    except BaseException:
+        # the body failed: put the stashed gradients back (dropping a half-made scaled one) and let the error through
+        for p in stash.all_fp32_from_fp32_params:
+            if id(p) in stashed_fp32:
+                p.grad = stashed_fp32[id(p)]
+        raise
     model_grads, master_grads = [], []
     if stash.master_grad_bucket is None and stash.all_fp32_from_fp16_params:
         masters = stash.all_fp32_from_fp16_params

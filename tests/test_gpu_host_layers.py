@@ -490,3 +490,19 @@ def test_zero_mode_trains_exactly_like_the_plain_mode(fused, fused_opt):
     for k in (0, 1):
         for a, b in zip(finals[False][k], finals[True][k]):
             assert_bits_equal(b[:a.numel()], a, "zero vs plain")
+
+
+def test_scale_loss_restores_stashed_gradients_when_the_body_raises():
+    torch.manual_seed(5)
+    model = torch.nn.Sequential(torch.nn.Linear(8, 8), torch.nn.BatchNorm1d(8)).to(DEV)
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    x = torch.randn(4, 8, device=DEV, dtype=torch.float16)
+    with amp.scale_loss(rm(x).float().sum(), opt) as scaled:
+        scaled.backward()
+    kept = model[1].weight.grad.clone()
+    with pytest.raises(RuntimeError, match="boom"):
+        with amp.scale_loss(rm(x).float().sum(), opt) as scaled:
+            raise RuntimeError("boom")
+    assert torch.equal(model[1].weight.grad, kept)
