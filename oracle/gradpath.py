@@ -30,10 +30,21 @@ in ``tests/test_oracle_pins.py``):
   per-tensor sums are accumulated in float64 and rounded to fp32 once; ATen's CPU
   fp32 accumulation (``per_tensor_norms_aten``) drifts by up to 1e-2 relative at
   these sizes and is only the timed baseline.
-* ``LossScalerState.update_scale`` (dynamic schedule) is OURS, not the
-  reference's: Apex's schedule is not in the reference tree -> parity unpinned
-  for the schedule itself; the rank-sharing wrapper ``patched_update_scale``
-  follows ``pyrannc/amp/__init__.py:44-65`` and is pinned by case analysis.
+* ``LossScalerState.update_scale``: Apex's published ``LossScaler.update_scale``
+  (``apex/amp/scaler.py`` at the pinned commit: halve on overflow, floor at
+  ``min_loss_scale``, zero the clean-step counter; otherwise count the step;
+  double, capped at ``max_loss_scale``, when the counter reaches ``scale_window``;
+  a static scale never skips) restated, and pinned by hand-written sequences of
+  (scale, counter, skip) literals.  The rank-sharing wrapper
+  ``patched_update_scale`` follows ``pyrannc/amp/__init__.py:44-65`` and is pinned
+  by case analysis.
+* ``reference_step_cpu`` (the timed CPU baseline): flag exact, norm to 1e-4 (it
+  sums in ATen's fp32) and bucket bit-exact given its own coefficient against
+  ``fused_step`` on a mixed list, an overflow case and a no-clip case.
+* Parity unpinned: only ``unscale_accumulate`` versus Apex's
+  ``multi_tensor_axpby`` (whether that kernel contracts multiply and add into one
+  fma is not visible from the reference tree); it is pinned against numpy's two
+  roundings instead.
 """
 from __future__ import annotations
 
@@ -348,25 +359,36 @@ def align_buffer(param: torch.Tensor, nranks: int) -> torch.Tensor:
 
 @dataclass
 class LossScalerState:
-    """Dynamic loss scale.  The schedule (halve on overflow, double after ``scale_window``
-    clean steps, clamped to [min, max]) is this project's own statement of the usual
-    dynamic-scaling policy; Apex's is not in the reference tree (parity unpinned)."""
+    """Apex ``LossScaler`` state and ``update_scale`` (external: ``apex/amp/scaler.py`` at the
+    commit pinned by ``docker/ubuntu/runtime/Dockerfile:13``; the reference reads and writes
+    ``_loss_scale`` / ``_unskipped`` and wraps ``update_scale``, ``pyrannc/amp/__init__.py:45-65``).
+    Published algorithm: on overflow with a dynamic scale the scale is halved (not below
+    ``min_loss_scale`` when one is given), the clean-step counter is zeroed and the step is
+    skipped; otherwise the counter is incremented; when the counter reaches ``scale_window``
+    the scale is doubled (not above ``max_loss_scale``) and the counter zeroed.  A static scale
+    never changes and never skips."""
     loss_scale: float = 2.0 ** 16
     unskipped: int = 0
     scale_window: int = 2000
-    min_loss_scale: float = 1.0
+    min_loss_scale: Optional[float] = None
     max_loss_scale: float = 2.0 ** 24
+    dynamic: bool = True
 
     def update_scale(self, had_overflow: bool) -> bool:
-        if had_overflow:
-            self.loss_scale = max(self.min_loss_scale, self.loss_scale / 2.0)
+        if had_overflow and self.dynamic:
+            should_skip = True
+            if self.min_loss_scale:
+                self.loss_scale = max(self.min_loss_scale, self.loss_scale / 2.0)
+            else:
+                self.loss_scale = self.loss_scale / 2.0
             self.unskipped = 0
         else:
+            should_skip = False
             self.unskipped += 1
-        if self.unskipped == self.scale_window:
+        if self.unskipped == self.scale_window and self.dynamic:
             self.loss_scale = min(self.max_loss_scale, self.loss_scale * 2.0)
             self.unskipped = 0
-        return had_overflow
+        return should_skip
 
 
 def patched_update_scale(state: LossScalerState, had_overflow_local: bool,

@@ -39,16 +39,20 @@ def test_make_grads_is_seeded_and_injects():
     assert a[0].dtype == torch.float16
 
 
-def test_loss_scaler_schedule_matches_the_stated_policy():
+def test_loss_scaler_schedule_literal_sequence():
+    """The product's scaler against hand-written literals (Apex's published schedule) and, step by
+    step, against the oracle's restatement of it."""
     ours = amp.LossScaler("dynamic", min_loss_scale=1.0, max_loss_scale=2.0 ** 10, scale_window=3)
     ours._loss_scale = 2.0 ** 8
     want = oracle.LossScalerState(loss_scale=2.0 ** 8, scale_window=3, min_loss_scale=1.0, max_loss_scale=2.0 ** 10)
     seq = [False, False, True, False, False, False, True, True, False, False, False, False, False, False, False]
-    for had in seq:
+    scales = [256, 256, 128, 128, 128, 256, 128, 64, 64, 64, 128, 128, 128, 256, 256]
+    counts = [1, 2, 0, 1, 2, 0, 0, 0, 1, 2, 0, 1, 2, 0, 1]
+    for had, scale, count in zip(seq, scales, counts):
         ours._has_overflow = had
-        assert ours.update_scale() == want.update_scale(had)
+        assert ours.update_scale() == had == want.update_scale(had)
         ours.clear_overflow_state()
-        assert (ours.loss_scale(), ours._unskipped) == (want.loss_scale, want.unskipped)
+        assert (ours.loss_scale(), ours._unskipped) == (scale, count) == (want.loss_scale, want.unskipped)
     static = amp.LossScaler(128.0)
     static._has_overflow = True
     assert static.update_scale() is False and static.loss_scale() == 128.0

@@ -299,6 +299,99 @@ def test_patched_update_scale_cases():
     assert oracle.patched_update_scale(s, False, other_flags=[1], other_scales=[512]) is True and s.loss_scale == 128
 
 
+def test_update_scale_hand_written_sequences():
+    """Apex's published schedule, pinned by literals worked out by hand (not by a second typing
+    of the formula): (had_overflow) -> (skip, loss_scale, unskipped) after the call."""
+    s = oracle.LossScalerState(loss_scale=256.0, scale_window=3, min_loss_scale=None, max_loss_scale=512.0)
+    steps = [
+        (True,  (True, 128.0, 0)),    # overflow: halve, counter to zero, skip
+        (False, (False, 128.0, 1)),
+        (False, (False, 128.0, 2)),
+        (False, (False, 256.0, 0)),   # third clean step in a row: double, counter to zero
+        (False, (False, 256.0, 1)),
+        (True,  (True, 128.0, 0)),    # an overflow forgets the clean steps counted so far
+        (True,  (True, 64.0, 0)),
+        (False, (False, 64.0, 1)),
+        (False, (False, 64.0, 2)),
+        (False, (False, 128.0, 0)),
+        (False, (False, 128.0, 1)),
+        (False, (False, 128.0, 2)),
+        (False, (False, 256.0, 0)),
+        (False, (False, 256.0, 1)),
+        (False, (False, 256.0, 2)),
+        (False, (False, 512.0, 0)),
+        (False, (False, 512.0, 1)),
+        (False, (False, 512.0, 2)),
+        (False, (False, 512.0, 0)),   # capped at max_loss_scale; the counter still restarts
+    ]
+    for i, (had, want) in enumerate(steps):
+        assert (s.update_scale(had), s.loss_scale, s.unskipped) == want, i
+    # floor: with min_loss_scale the scale stops there, without one it keeps halving below 1
+    s = oracle.LossScalerState(loss_scale=4.0, min_loss_scale=2.0)
+    assert [(s.update_scale(True), s.loss_scale) for _ in range(3)] == [(True, 2.0), (True, 2.0), (True, 2.0)]
+    s = oracle.LossScalerState(loss_scale=2.0, min_loss_scale=None)
+    assert [(s.update_scale(True), s.loss_scale) for _ in range(3)] == [(True, 1.0), (True, 0.5), (True, 0.25)]
+    # defaults of amp.initialize: 2^16 start, 2000-step window, 2^24 cap
+    s = oracle.LossScalerState()
+    assert (s.loss_scale, s.scale_window, s.max_loss_scale, s.min_loss_scale) == (65536.0, 2000, 16777216.0, None)
+    for _ in range(1999):
+        assert s.update_scale(False) is False
+    assert (s.loss_scale, s.unskipped) == (65536.0, 1999)
+    assert s.update_scale(False) is False and (s.loss_scale, s.unskipped) == (131072.0, 0)
+    # a static scale neither moves nor skips, overflow or not
+    s = oracle.LossScalerState(loss_scale=128.0, dynamic=False, scale_window=2)
+    assert [s.update_scale(h) for h in (True, False, True, False)] == [False] * 4 and s.loss_scale == 128.0
+
+
+# ----------------------------------------------------------------------------- timed CPU baseline
+
+def _bucket_views(grads, dtype):
+    n = sum(g.numel() for g in grads)
+    bucket = torch.full((n,), 7.0, dtype=dtype)        # stale values: every element must be overwritten
+    views, off = [], 0
+    for g in grads:
+        views.append(bucket.narrow(0, off, g.numel()).view(g.shape))
+        off += g.numel()
+    return bucket, views
+
+
+@pytest.mark.parametrize("src_dtype,inv_scale", [(torch.bfloat16, 2.0 ** -16), (torch.float16, 2.0 ** -12),
+                                                 (torch.float32, 1.0)])
+def test_reference_step_cpu_does_the_work_of_fused_step(src_dtype, inv_scale):
+    """The timed CPU leg against the oracle's fused step on the same mixed list: flag exact,
+    norm within 1e-4 (ATen's fp32 accumulation), coefficient consistent with its own norm, and
+    the bucket it leaves bit-exact given that coefficient."""
+    gen = torch.Generator().manual_seed(11)
+    shapes = [(257, 33), (1,), (4096,), (3, 5, 7), (0,), (63,), (1000, 17)]
+    grads = [(torch.randn(s, generator=gen) * 1e-2 / inv_scale).to(src_dtype) for s in shapes]
+    for max_norm in (1.0, 1e6):                        # clips / does not clip
+        bucket, views = _bucket_views(grads, torch.float32)
+        ovf, norm, coef = oracle.reference_step_cpu(grads, views, inv_scale, max_norm)
+        want = oracle.fused_step(grads, ["f32"] * len(grads), inv_scale, max_norm)
+        assert ovf == want.overflow == 0
+        assert math.isclose(norm, want.norm, rel_tol=1e-4)
+        assert (coef is None) == (want.coef is None) == (max_norm == 1e6)
+        unscaled = oracle.fused_step(grads, ["f32"] * len(grads), inv_scale, math.inf).buckets["f32"]
+        if coef is not None:
+            assert math.isclose(coef, want.coef, rel_tol=1e-4)
+            assert coef == float(np.float32(max_norm)) / (norm + 1e-6)
+            unscaled = (unscaled.numpy() * np.float32(coef)).astype(np.float32)
+            assert np.array_equal(f32_bits(bucket), unscaled.view(np.uint32))
+        else:
+            assert np.array_equal(f32_bits(bucket), f32_bits(unscaled))
+    # overflow: flagged, nothing clipped (the step is skipped)
+    bad = [g.clone() for g in grads]
+    bad[3].view(-1)[104] = float("inf")
+    bad[6].view(-1)[0] = float("nan")
+    bucket, views = _bucket_views(bad, torch.float32)
+    ovf, norm, coef = oracle.reference_step_cpu(bad, views, inv_scale, 1.0)
+    want = oracle.fused_step(bad, ["f32"] * len(bad), inv_scale, 1.0)
+    assert ovf == want.overflow == 1 and coef is None and want.coef is None
+    finite = torch.isfinite(bucket)
+    assert int((~finite).sum()) == 2
+    assert torch.equal(bucket[finite], want.buckets["f32"][finite])     # written unscaled, unclipped
+
+
 # ----------------------------------------------------------------------------- accumulation
 
 def test_unscale_accumulate_is_two_roundings():
