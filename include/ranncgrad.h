@@ -198,6 +198,22 @@ int rg_tensor_norms_device_ptr(const rg_plan* plan, const float** out_dev);
 int rg_read_result(rg_plan* plan, rg_step_result* out_host, void* stream);
 int rg_read_tensor_norms(rg_plan* plan, float* out_host, void* stream);
 
+/* The fused step of rg_fused_step for ONE tensor pair, without a plan and without allocating
+ * anything.  It has no counterpart in the reference; it is for callers that cannot call
+ * hipMalloc or rg_plan_create: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid allocation.  The working memory a plan would own (result block, per-chunk
+ * partial sums) is a fixed array of about 3 MiB in the library's device image, one copy per
+ * GPU, held until the process ends; numel above RG_STATIC_MAX_NUMEL is rejected with
+ * RG_EINVAL.  The kernels overwrite every slot they later read, so nothing needs clearing
+ * between calls; calls that overlap on one GPU (two streams, two threads) race on that array
+ * and must be serialised by the caller.  Same arithmetic, same launch shapes and therefore
+ * the same bits as rg_fused_step on a one-tensor plan; `result_dev` (device memory of the
+ * caller, 8-byte aligned, may be NULL) receives the rg_step_result on the stream. */
+#define RG_STATIC_MAX_NUMEL 4294967296LL /* 2^32 elements */
+int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t numel, int src_dtype, int dst_dtype,
+                         float inv_scale, float max_norm, int flags, rg_step_result* result_dev, int device,
+                         void* stream);
+
 /* ---------------------------------------------------------------- optimizer step */
 
 /* Multi-tensor optimizer step on fp32 parameters, the step that follows the clip: the

@@ -65,6 +65,7 @@ SIGNATURES = {
     "rg_grad_norm": (_i, [_vp, _vp]),
     "rg_scale_cast": (_i, [_vp, _f, _vp]),
     "rg_scale_cast_single": (_i, [_vp, _vp, _i64, _i, _i, _f, _i, _vp]),
+    "rg_fused_step_static": (_i, [_vp, _vp, _i64, _i, _i, _f, _f, _i, _vp, _i, _vp]),
     "rg_zero": (_i, [_vp, _vp]),
     "rg_fill_zero": (_i, [_vp, _i64, _i, _vp]),
     "rg_result_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
@@ -266,6 +267,16 @@ def scale_cast_single(src_ptr: Optional[int], dst_ptr: int, numel: int, src_dtyp
                       scale: float, device: int, stream: int = 0) -> None:
     check(lib.rg_scale_cast_single(_vp(src_ptr or None), _vp(dst_ptr or None), numel, src_dtype, dst_dtype,
                                    scale, device, _vp(stream)))
+
+
+RG_STATIC_MAX_NUMEL = 1 << 32
+
+
+def fused_step_static(src_ptr: int, dst_ptr: int, numel: int, src_dtype: int, dst_dtype: int, inv_scale: float,
+                      max_norm: float, flags: int, result_ptr: Optional[int], device: int, stream: int = 0) -> None:
+    """The fused step over one tensor pair with no plan and no allocation (``rg_fused_step_static``)."""
+    check(lib.rg_fused_step_static(_vp(src_ptr or None), _vp(dst_ptr or None), numel, src_dtype, dst_dtype, inv_scale,
+                                   max_norm, flags, _vp(result_ptr or None), device, _vp(stream)))
 
 
 def fill_zero(ptr: int, nbytes: int, device: int, stream: int = 0) -> None:

@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -406,6 +407,7 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
 
 static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_overflow) {
   FinalizeArgs f;
+  memset(&f, 0, sizeof(f));
   f.tensor_chunk_begin = p->d_tensor_chunk_begin;
   f.chunk_sumsq = p->d_chunk_sumsq;
   f.chunk_bad = p->d_chunk_bad;
@@ -668,6 +670,125 @@ RG_API int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t nume
   DeviceGuard guard(device);
   const bool streaming = numel * (ss + ds) > ((int64_t)256 << 20);
   RG_HIP(launch_pass(kModeWrite, a, streaming, reinterpret_cast<hipStream_t>(stream)));
+  return RG_OK;
+}
+
+// ---------------------------------------------------------------------------- allocation-free fused step
+
+// Working memory of rg_fused_step_static: what a plan keeps in its own allocation (result
+// block, per-tensor norm, one partial sum and flag per chunk), for one tensor pair of at most
+// RG_STATIC_MAX_NUMEL elements.  Every GPU the library runs on holds its own copy of this
+// array until the process ends; host code only ever uses the per-device address looked up below.
+constexpr int64_t kStaticMaxChunks = RG_STATIC_MAX_NUMEL / RG_DEFAULT_CHUNK_ELEMS;
+constexpr size_t kStaticResultOff = 0;        // StepResult
+constexpr size_t kStaticTensorOff = 256;      // float norm @0, double sq @8, int32 bad @16
+constexpr size_t kStaticSumsqOff = 512;       // double[kStaticMaxChunks]
+constexpr size_t kStaticBadOff = kStaticSumsqOff + (size_t)kStaticMaxChunks * sizeof(double);
+constexpr size_t kStaticScratchBytes = kStaticBadOff + (size_t)kStaticMaxChunks * sizeof(int32_t);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static char* g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch` on each GPU, looked up once
+
+// The address of this GPU's copy of `scratch` (the caller has made `device` current).
+static int static_scratch(int device, char** out) {
+  if (device < 0 || device >= kMaxDevices) {
+    set_error("rg_fused_step_static: device %d is outside [0, %d)", device, kMaxDevices);
+    return RG_EINVAL;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    RG_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[device] = static_cast<char*>(ptr);
+  }
+  *out = g_scratch_ptr[device];
+  return RG_OK;
+}
+
+RG_API int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t numel, int src_dtype, int dst_dtype,
+                                float inv_scale, float max_norm, int flags, rg_step_result* result_dev, int device,
+                                void* stream) {
+  const int ss = elem_size(src_dtype), ds = elem_size(dst_dtype);
+  if (ss < 0 || ds < 0 || numel < 0 || (numel > 0 && (src_dev == nullptr || dst_dev == nullptr))) {
+    set_error("rg_fused_step_static: bad arguments (dtypes %d->%d, numel %lld)", src_dtype, dst_dtype, (long long)numel);
+    return RG_EINVAL;
+  }
+  if (numel > (int64_t)RG_STATIC_MAX_NUMEL) {
+    set_error("rg_fused_step_static: %lld elements exceed the limit of %lld; use a plan (rg_fused_step)",
+              (long long)numel, (long long)RG_STATIC_MAX_NUMEL);
+    return RG_EINVAL;
+  }
+  if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
+    set_error("rg_fused_step_static: inv_scale must be a non-zero number");
+    return RG_EINVAL;
+  }
+  int rc = check_pointer(src_dev, ss, "src", 0);
+  if (rc == RG_OK) rc = check_pointer(dst_dev, ds, "dst", 0);
+  if (rc == RG_OK) rc = check_pointer(result_dev, 8, "result", 0);
+  if (rc != RG_OK) return rc;
+  if (src_dev == dst_dev && src_dtype != dst_dtype) {
+    set_error("rg_fused_step_static: in place but changes dtype");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(device);
+  char* base = nullptr;
+  rc = static_scratch(device, &base);
+  if (rc != RG_OK) return rc;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+
+  // the launch shapes of a one-tensor plan, so that both give the same bits
+  const int64_t chunk = default_chunk_elems(numel);
+  const int64_t n_chunks = (numel + chunk - 1) / chunk;
+  const bool streaming = numel * (ss + ds) > ((int64_t)256 << 20);
+  const int64_t head = numel > 0 ? tensor_head(src_dev, dst_dev, ss, ds) : 0;
+  const bool offgrid = numel > head &&
+      ((reinterpret_cast<uintptr_t>(src_dev) + (uintptr_t)(head * ss)) & (kAlignBytes - 1)) != 0;
+
+  PassArgs a;
+  memset(&a, 0, sizeof(a));
+  a.single.src = src_dev;
+  a.single.dst = dst_dev;
+  a.single.src_dtype = (int16_t)src_dtype;
+  a.single.dst_dtype = (int16_t)dst_dtype;
+  a.single_numel = numel;
+  a.single_chunk_elems = chunk;
+  a.single_head = head;
+  a.peel_heads = head != 0 ? 1 : 0;
+  a.chunk_sumsq = reinterpret_cast<double*>(base + kStaticSumsqOff);
+  a.chunk_bad = reinterpret_cast<int32_t*>(base + kStaticBadOff);
+  a.n_chunks = n_chunks;
+  a.tile_elems = (int32_t)chunk;
+  a.tiles_per_chunk = 1;
+  a.scale = inv_scale;
+  a.xcd_run = 64;
+  RG_HIP(launch_pass(kModeReduce, a, streaming, s));
+
+  FinalizeArgs f;
+  memset(&f, 0, sizeof(f));
+  f.single_chunks = n_chunks;
+  f.chunk_sumsq = a.chunk_sumsq;
+  f.chunk_bad = a.chunk_bad;
+  f.tensor_norm = reinterpret_cast<float*>(base + kStaticTensorOff);
+  f.tensor_sq = reinterpret_cast<double*>(base + kStaticTensorOff + 8);
+  f.tensor_bad = reinterpret_cast<int32_t*>(base + kStaticTensorOff + 16);
+  f.result = reinterpret_cast<StepResult*>(base + kStaticResultOff);
+  f.result_copy = result_dev;
+  f.n_tensors = 1;
+  f.max_norm = max_norm;
+  f.ignore_overflow = (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0;
+  f.partials_per_chunk = 1;
+  RG_HIP(launch_finalize(f, s));
+
+  a.result = f.result;
+  a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
+  a.xcd_run = offgrid ? 256 : 0;
+  if (kWriteTileElems < chunk) {
+    a.tile_elems = kWriteTileElems;
+    a.tiles_per_chunk = (int32_t)((chunk + kWriteTileElems - 1) / kWriteTileElems);
+  }
+  RG_HIP(launch_pass(kModeWrite, a, streaming, s));
   return RG_OK;
 }
 

@@ -118,13 +118,15 @@ struct PassArgs {
 };
 
 struct FinalizeArgs {
-  const int64_t* tensor_chunk_begin;  // [n_tensors + 1]
+  const int64_t* tensor_chunk_begin;  // [n_tensors + 1]; null = one tensor made of `single_chunks` chunks
+  int64_t single_chunks;
   const double* chunk_sumsq;
   const int32_t* chunk_bad;
   float* tensor_norm;                 // [n_tensors]
   double* tensor_sq;                  // [n_tensors]
   int32_t* tensor_bad;                // [n_tensors]
   StepResult* result;
+  rg_step_result* result_copy;        // optional second place the decision is written to (caller's memory)
   int32_t n_tensors;
   float max_norm;
   int32_t ignore_overflow;  // overflow is reported but neither gates the clip nor the write

@@ -362,8 +362,9 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_tensors_kernel(Finaliz
   double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
   int bad = 0;
   // partials_per_chunk > 1: the pass left one partial per tile, laid out chunk-major
-  const int64_t end = a.tensor_chunk_begin[t + 1] * a.partials_per_chunk;
-  int64_t c = a.tensor_chunk_begin[t] * a.partials_per_chunk + threadIdx.x;
+  const int64_t first = a.tensor_chunk_begin ? a.tensor_chunk_begin[t] : 0;
+  const int64_t end = (a.tensor_chunk_begin ? a.tensor_chunk_begin[t + 1] : a.single_chunks) * a.partials_per_chunk;
+  int64_t c = first * a.partials_per_chunk + threadIdx.x;
   for (; c + 3 * kBlockThreads < end; c += 4 * kBlockThreads) {
     const double v0 = a.chunk_sumsq[c], v1 = a.chunk_sumsq[c + kBlockThreads];
     const double v2 = a.chunk_sumsq[c + 2 * kBlockThreads], v3 = a.chunk_sumsq[c + 3 * kBlockThreads];
@@ -419,6 +420,13 @@ __global__ __launch_bounds__(kBlockThreads) void finalize_total_kernel(FinalizeA
     a.result->overflow = overflow;
     a.result->clipped = clip ? 1 : 0;
     a.result->skipped = gate ? 1 : 0;
+    if (a.result_copy != nullptr) {
+      a.result_copy->norm = norm;
+      a.result_copy->coef = clip ? (float)((double)a.max_norm / g) : 1.0f;
+      a.result_copy->overflow = overflow;
+      a.result_copy->clipped = clip ? 1 : 0;
+      a.result_copy->skipped = gate ? 1 : 0;
+    }
   }
 }
 
