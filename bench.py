@@ -1,13 +1,17 @@
 #!/usr/bin/env python3
-"""Benchmark of the fused unscale + overflow-check + norm + clip + pack step on one MI355X.
+"""Benchmark of the per-step parameter/gradient path on one MI355X.
 
-A "step" is one pass of the fused step over one batch of synthetic gradients that are already
-resident in HBM: pass 1 reads the gradients (flag + per-tensor sums of squares), a small
-kernel derives the global norm and the clip coefficient on the device, pass 2 re-reads the
-gradients and writes the unscaled, clipped values into the packed fp32 bucket.
+A "step" is one pass of the measured operation over one batch of synthetic tensors that are already
+resident in HBM.  The headline operation is the fused step - pass 1 reads the gradients (inf/NaN
+flag + per-tensor sums of squares), a small kernel derives the global norm and the clip coefficient
+on the device, pass 2 re-reads the gradients and writes the unscaled, clipped values into the packed
+bucket - on the largest configuration that fits one GPU, ``c3_bert_enlarged``.
 
-Prints ONE JSON line.  `value` is algorithmic GB/s over the whole step: (2*s + d) * N bytes
-(s, d = source / destination bytes per element) divided by the measured time per step.
+Prints ONE JSON line.  ``value`` is algorithmic GB/s over the whole step: the bytes the operation must
+move (``(2s + d) N`` for a fused step that clips; s, d = source / destination bytes per element) divided
+by the wall time per step.  With no ``--workload`` / ``--op`` the line also carries ``configs``: the same
+measurement for every other configuration and operation of the path (each can be run alone with
+``--workload`` / ``--op``, which is how the profiles under ``profiles/`` are made).
 """
 from __future__ import annotations
 
@@ -15,30 +19,33 @@ import argparse
 import json
 import os
 import platform
+import re
 import sys
 import time
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+ROOT = os.path.dirname(os.path.abspath(__file__))
+HEADLINE = "c3_bert_enlarged"
 
-# HBM traffic per launch of the dominant kernel (the write pass), from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs of this same command, each scaled by what the counter reads for
-# a plain 1 GiB copy (profiles/fused_step_c2_bert_large_hbm_traffic.txt).  Missing = not measured.
-MEASURED_TRAFFIC_BYTES = {"c2_bert_large": 2021548222}
-# the Adam step with bf16 model copy, same method (profiles/adam_step_c2_bert_large_kernel_stats.txt)
-MEASURED_TRAFFIC_BYTES_ADAM = {"c2_bert_large": 10075311450}
+FUSED_OPS = ("fused_step", "fused_step_noclip", "fused_step_noclip_2pass", "overflow_host_gate", "unscale_pack",
+             "copy_back", "unflatten_back", "grad_norm", "zero")
+C5_OPS = ("c5_unflatten", "c5_master_cast", "c5_copy_back", "c5_repack")
+OPTIM_OPS = ("adam", "sgd", "adam_from_model_grads")
+ALL_OPS = ("all",) + FUSED_OPS + C5_OPS + OPTIM_OPS
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2_bert_large")
-    ap.add_argument("--op", default="fused_step", choices=["fused_step", "adam", "sgd", "adam_from_model_grads"],
-                    help="fused_step (default: the graded metric), the optimizer step that follows it, or both "
-                         "without ever writing the unscaled gradients (read pass + clip decision + Adam reading the scaled grads)")
+    ap.add_argument("--workload", default=None,
+                    help="c1_mlp | c2_bert_large | c3_bert_enlarged | c3_bert_enlarged_overflow | c4_resnet152x2 | c5_zero_flat")
+    ap.add_argument("--op", default=None, choices=ALL_OPS,
+                    help="all (default: headline + every configuration), or one operation to run alone")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--chunk-elems", type=int, default=0)
+    ap.add_argument("--c5-elements", type=int, default=10_000_000_000, help="total elements of the ZeRO flat buffer")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 1 GiB fp32 tensor copies first (known traffic, for scaling "
@@ -58,21 +65,308 @@ def cpu_model() -> str:
     return platform.processor() or "unknown"
 
 
-def cpu_baseline(cfg, seed: int, budget_s: float):
-    """The reference's op sequence on the host cores (oracle.reference_step_cpu), on a bounded
-    sample of the same workload: the same tensor list with dim 0 of every tensor scaled so
-    that one CPU step fits the budget several times."""
+# ----------------------------------------------------------------------------- measured traffic
+
+def measured_traffic(op: str, workload: str, kernel: str):
+    """HBM bytes per launch of ``kernel`` from the committed rocprofv3 --pmc summary of this operation and
+    workload (``profiles/<op>_<workload>_hbm_traffic.txt``, lines ``traffic_bytes_per_launch: <kernel> = <bytes>``),
+    or None when that summary does not exist."""
+    path = os.path.join(ROOT, "profiles", f"{op}_{workload}_hbm_traffic.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                m = re.match(r"traffic_bytes_per_launch:\s*(.+?)\s*=\s*([0-9]+)\s*$", line)
+                if m and m.group(1) == kernel:
+                    return int(m.group(2))
+    except OSError:
+        pass
+    return None
+
+
+# ----------------------------------------------------------------------------- timing
+
+def timed(fn, steps: int, warmup: int, min_untimed: int = 0):
+    """warm-up (at least ``min_untimed`` untimed calls so the clocks have ramped), then exactly ``steps`` calls
+    between two synchronisations.  Returns (wall seconds per step, device seconds per step from events on the
+    launch stream, which is torch's current stream for every kernel of the library)."""
+    import torch
+    for _ in range(max(min_untimed, warmup)):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    while not e1.query():             # poll: a blocking wait adds its wake-up latency to the last step
+        pass
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    return wall, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def roofline(kernel: str, bytes_per_launch: int, launch_s: float, traffic, **extra) -> dict:
+    achieved = bytes_per_launch / launch_s / 1e9
+    out = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+           "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+           "algorithmic_bytes_per_launch": int(bytes_per_launch), "avg_launch_ms": round(launch_s * 1e3, 4)}
+    out.update(extra)
+    return out
+
+
+def entry(workload: str, op: str, step_s: float, step_bytes: int, roof: dict, **extra) -> dict:
+    gbps = step_bytes / step_s / 1e9
+    out = {"workload": workload, "op": op, "ms_per_step": round(step_s * 1e3, 4), "algorithmic_bytes_per_step": int(step_bytes),
+           "GB/s": round(gbps, 1), "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2), "roofline": roof}
+    out.update(extra)
+    return out
+
+
+# ----------------------------------------------------------------------------- fused-step workloads
+
+class StepWorkload:
+    """Gradients of one configuration on the device, with the packed destination bucket and its views."""
+
+    def __init__(self, key: str, seed: int, chunk_elems: int = 0):
+        import torch
+        from rannc_amd.multi_tensor import TensorPlan
+        from rannc_amd.workloads import make_grads, step_config
+        self.torch, self.key = torch, key
+        self.cfg = step_config(key)
+        self.dev = torch.device("cuda", 0)
+        self.grads, _ = make_grads(self.cfg, seed, device=str(self.dev))
+        self.n = sum(g.numel() for g in self.grads)
+        self.ddt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[self.cfg.bucket_dtype]
+        self.bucket = torch.zeros(self.n, dtype=self.ddt, device=self.dev)
+        self.views, off = [], 0
+        for g in self.grads:
+            self.views.append(self.bucket.narrow(0, off, g.numel()))
+            off += g.numel()
+        self.s, self.d = self.grads[0].element_size(), self.bucket.element_size()
+        self.plan = TensorPlan(self.grads, self.views, chunk_elems=chunk_elems)
+
+    def close(self):
+        self.plan.close()
+        self.grads = self.views = self.bucket = None
+        self.torch.cuda.empty_cache()
+
+    def describe(self) -> dict:
+        return {"workload": self.key, "description": self.cfg.description, "tensors": len(self.grads), "elements": self.n,
+                "src_bytes_per_elem": self.s, "dst_bytes_per_elem": self.d,
+                "chunk_elems": self.plan.plan.chunk_elems, "chunks": self.plan.plan.num_chunks}
+
+
+def run_fused_step(w: StepWorkload, steps: int, warmup: int, op: str = "fused_step") -> dict:
+    """The fused step.  ``op`` selects the strategy: the default two passes, ``fused_step_noclip`` = a bound the norm
+    stays under with the one-pass strategy asked for (RG_STEP_EXPECT_NO_CLIP), ``fused_step_noclip_2pass`` = the same
+    bound with the default two passes."""
+    from rannc_amd import _lib
+    torch, cfg, plan = w.torch, w.cfg, w.plan
+    max_norm = cfg.max_norm if op == "fused_step" else 1e30
+    flags = _lib.RG_STEP_EXPECT_NO_CLIP if op == "fused_step_noclip" else _lib.RG_STEP_DEFAULT
+
+    def step():
+        plan.fused_step(cfg.inv_scale, max_norm, flags)
+
+    # Untimed: the warm-up steps asked for, preceded by enough further steps that the GPU has left its idle clocks.
+    for _ in range(max(60, warmup)):
+        step()
+    torch.cuda.synchronize()
+    # Timed region: HIP events (recorded by the library on the launch stream) bracket only the last kernel of the
+    # step - the dominant one - and only on every fifth step: each record costs a few microseconds of stream time.
+    stride = min(5, max(1, steps))
+    sampled = (steps + stride - 1) // stride
+    plan.plan.enable_timing(-sampled)
+    plan.plan.timing_stride(stride)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    done = torch.cuda.Event()
+    done.record()
+    while not done.query():
+        pass
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / steps
+    res = plan.result()
+    last_only = [plan.plan.read_timing(i) for i in range(sampled)]
+    plan.plan.timing_stride(1)
+    # A second, untimed loop brackets all stages for the breakdown.
+    k = min(steps, 50)
+    plan.plan.enable_timing(k)
+    for _ in range(k):
+        step()
+    torch.cuda.synchronize()
+    per_kernel = [plan.plan.read_timing(i) for i in range(k)]
+    plan.plan.enable_timing(0)
+
+    n, s, d = w.n, w.s, w.d
+    clipped, overflow = bool(res.clipped), int(res.overflow)
+    last_ms = sum(x[2] for x in last_only) / len(last_only)
+    first_ms = sum(x[0] for x in per_kernel) / len(per_kernel)
+    mid_ms = sum(x[1] for x in per_kernel) / len(per_kernel)
+    extra = {}
+    if op == "fused_step_noclip":
+        # one pass (read s, write d) + decision + a gated in-place scale kernel that finds nothing to do
+        step_bytes = (s + d) * n
+        roof = roofline("pass_kernel<reduce+write, streaming>", (s + d) * n, first_ms * 1e-3,
+                        measured_traffic(op, w.key, "pass_kernel<reduce+write>"),
+                        note="dominant kernel timed in a second, untimed loop with every stage bracketed",
+                        other_kernels={"combine_tiles+finalize_tensors+finalize_total": {"avg_launch_ms": round(mid_ms, 4)},
+                                       "pass_kernel<write> gated on the decision (idle)": {"avg_launch_ms": round(last_ms, 4)}})
+    else:
+        moved = s * n if (overflow and not clipped and res.skipped) else ((2 * s + d) * n if clipped else (s + d) * n)
+        step_bytes = (2 * s + d) * n if clipped else (s + d) * n
+        if res.skipped:
+            # the write pass is launched and finds the step skipped: it moves nothing
+            extra["bytes_moved_per_step"] = moved
+            extra["GB/s_on_bytes_moved"] = round(moved / step_s / 1e9, 1)
+            extra["pct_of_hbm_peak_on_bytes_moved"] = round(100.0 * moved / step_s / 1e9 / HBM_PEAK_GBPS, 2)
+            roof = roofline("pass_kernel<reduce, streaming>", s * n, first_ms * 1e-3,
+                            measured_traffic(op, w.key, "pass_kernel<reduce>"),
+                            note="the write pass found the step skipped; its idle launch took %.1f us" % (last_ms * 1e3),
+                            other_kernels={"pass_kernel<write> (skipped on the device)": {"avg_launch_ms": round(last_ms, 4)},
+                                           "finalize_tensors+finalize_total": {"avg_launch_ms": round(mid_ms, 4)}})
+        else:
+            roof = roofline("pass_kernel<write, streaming>", (s + d) * n, last_ms * 1e-3,
+                            measured_traffic(op, w.key, "pass_kernel<write>"), launches_timed=len(last_only),
+                            other_kernels={
+                                "pass_kernel<reduce>": {"avg_launch_ms": round(first_ms, 4), "algorithmic_bytes_per_launch": s * n,
+                                                        "achieved": round(s * n / (first_ms * 1e-3) / 1e9, 1),
+                                                        "traffic": measured_traffic(op, w.key, "pass_kernel<reduce>")},
+                                "finalize_tensors+finalize_total": {"avg_launch_ms": round(mid_ms, 4)},
+                                "note": "from a second, untimed loop of the same steps with all stages bracketed"})
+    return entry(w.key, op, step_s, step_bytes, roof, clipped=clipped, overflow=overflow, skipped=int(res.skipped),
+                 norm=res.norm, coef=res.coef, steps=steps, elements_per_s=round(n / step_s, 1), **extra)
+
+
+def run_overflow_host_gate(w: StepWorkload, steps: int, warmup: int) -> dict:
+    """The two-call form a loss scaler uses: read pass, flag read on the host (it decides the loss scale there,
+    ``pyrannc/amp/__init__.py:44-65``), and the write pass only launched when the step is not skipped."""
+    cfg, plan = w.cfg, w.plan
+    state = {"res": None}
+
+    def step():
+        plan.step_begin(cfg.inv_scale)
+        state["res"] = plan.result()          # waits for the read pass
+        if not state["res"].overflow:
+            plan.step_finish(cfg.max_norm)
+
+    wall, dev_s = timed(step, steps, warmup, 20)
+    res = state["res"]
+    n, s, d = w.n, w.s, w.d
+    moved = s * n if res.overflow else (2 * s + d) * n
+    roof = roofline("pass_kernel<reduce, streaming>", s * n, dev_s, measured_traffic("overflow_host_gate", w.key, "pass_kernel<reduce>"),
+                    note="launch time = whole step from device events (read pass + finalize + the host's read of the flag)")
+    return entry(w.key, "overflow_host_gate", wall, moved, roof, overflow=int(res.overflow), steps=steps,
+                 note="bytes = what the step moves: s*N when it is skipped")
+
+
+def run_plan_op(w: StepWorkload, op: str, steps: int, warmup: int) -> dict:
+    """Single-kernel operations over the workload's tensor list."""
+    import torch
+    from rannc_amd.multi_tensor import TensorPlan
+    n, s, d = w.n, w.s, w.d
+    cleanup = []
+    if op == "unscale_pack":
+        fn, nbytes, kernel = (lambda: w.plan.unscale_pack(w.cfg.inv_scale)), (s + d) * n, "pass_kernel<reduce+write>"
+    elif op == "grad_norm":
+        fn, nbytes, kernel = w.plan.grad_norm, s * n, "pass_kernel<reduce>"
+    elif op == "zero":
+        fn, nbytes, kernel = w.plan.zero, d * n, "pass_kernel<write> (zero fill)"
+    elif op == "copy_back":
+        # fp32 masters (the packed bucket holds fp32 values after a step) -> model parameters in the gradient dtype
+        mdt = w.grads[0].dtype if w.grads[0].dtype != torch.float32 else torch.bfloat16
+        masters = torch.randn(n, device=w.dev, dtype=torch.float32)
+        mviews, off = [], 0
+        for g in w.grads:
+            mviews.append(masters.narrow(0, off, g.numel()))
+            off += g.numel()
+        models = [torch.empty(g.shape, dtype=mdt, device=w.dev) for g in w.grads]
+        plan = TensorPlan(mviews, models)
+        cleanup.append(plan)
+        fn, nbytes, kernel = (lambda: plan.scale_cast(1.0)), (4 + models[0].element_size()) * n, "pass_kernel<write>"
+    elif op == "unflatten_back":
+        # packed bucket -> one separately allocated tensor per parameter, same dtype
+        outs = [torch.empty(g.shape, dtype=w.ddt, device=w.dev) for g in w.grads]
+        plan = TensorPlan(w.views, outs)
+        cleanup.append(plan)
+        fn, nbytes, kernel = (lambda: plan.scale_cast(1.0)), 2 * d * n, "pass_kernel<write>"
+    else:
+        raise ValueError(op)
+    wall, dev_s = timed(fn, steps, warmup, 20)
+    for p in cleanup:
+        p.close()
+    extra = {}
+    if op == "unscale_pack":
+        extra["note"] = "launch time = pass + combine_tiles + finalize kernels (whole operation, device events)"
+    return entry(w.key, op, wall, nbytes, roofline(kernel, nbytes, dev_s, measured_traffic(op, w.key, kernel), **extra), steps=steps)
+
+
+# ----------------------------------------------------------------------------- ZeRO flat buffer (config 5)
+
+class ZeroFlat:
+    """fp16 flat buffer cut into 4096 odd-sized segments at odd offsets, separately allocated fp16 parameters and
+    fp32 masters (``DistributedParamLocator`` store / setScalarType / load at one rank)."""
+
+    def __init__(self, total: int, seed: int):
+        import torch
+        from rannc_amd.workloads import zero_segment_sizes
+        self.torch = torch
+        dev = torch.device("cuda", 0)
+        self.sizes = zero_segment_sizes(4096, total, seed=seed)
+        self.n = n = sum(self.sizes)
+        self.flat = torch.empty(n, dtype=torch.float16, device=dev)
+        step = 1 << 28
+        for lo in range(0, n, step):      # cheap on-device pattern: every fp16 bit pattern except inf / NaN
+            hi = min(n, lo + step)
+            idx = torch.arange(lo, hi, device=dev, dtype=torch.int64)
+            bits = ((idx * 2654435761) >> 7) & 0xFFFF
+            bits = torch.where((bits & 0x7C00) == 0x7C00, bits & 0x83FF, bits)
+            self.flat[lo:hi] = bits.to(torch.int16).view(torch.float16)
+            del idx, bits
+        offs = [0]
+        for sz in self.sizes:
+            offs.append(offs[-1] + sz)
+        self.flat_views = [self.flat.narrow(0, o, sz) for o, sz in zip(offs, self.sizes)]
+        self.params = [torch.empty(sz, dtype=torch.float16, device=dev) for sz in self.sizes]
+        self.masters = [torch.empty(sz, dtype=torch.float32, device=dev) for sz in self.sizes]
+
+    def close(self):
+        self.flat = self.flat_views = self.params = self.masters = None
+        self.torch.cuda.empty_cache()
+
+
+def run_c5(z: ZeroFlat, op: str, steps: int, warmup: int) -> dict:
+    from rannc_amd.multi_tensor import TensorPlan
+    src, dst, bpe = {"c5_unflatten": (z.flat_views, z.params, 4), "c5_master_cast": (z.params, z.masters, 6),
+                     "c5_copy_back": (z.masters, z.params, 6), "c5_repack": (z.params, z.flat_views, 4)}[op]
+    plan = TensorPlan(src, dst)
+    wall, dev_s = timed(lambda: plan.scale_cast(1.0), steps, warmup, 5)
+    plan.close()
+    nbytes = bpe * z.n
+    return entry("c5_zero_flat", op, wall, nbytes,
+                 roofline("pass_kernel<write, streaming>", nbytes, dev_s, measured_traffic(op, "c5_zero_flat", "pass_kernel<write>")),
+                 steps=steps, elements=z.n, segments=len(z.sizes))
+
+
+# ----------------------------------------------------------------------------- CPU baseline
+
+def cpu_baseline(key: str, seed: int, budget_s: float):
+    """The reference's op sequence on the host cores (oracle.reference_step_cpu), on a bounded sample of the same
+    workload: the same tensor list with dim 0 of every tensor scaled so that one CPU step fits the budget."""
     import torch
     from oracle import gradpath as oracle
-    from rannc_amd.workloads import make_grads
+    from rannc_amd.workloads import make_grads, step_config
 
+    cfg = step_config(key)
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
     torch.set_num_threads(threads)
     frac = 1.0
-    # ~0.3 GB/s per thread is a safe lower bound for the per-tensor op chain
-    est = cfg.total_numel * 8 / (0.3e9 * threads)
-    if est > budget_s / 4:
-        frac = max(0.02, (budget_s / 4) / est)
+    est = cfg.total_numel * 8 / (0.3e9 * threads)      # ~0.3 GB/s per thread is a safe lower bound for the op chain
+    if est > budget_s / 5:
+        frac = max(0.01, (budget_s / 5) / est)
     grads, _ = make_grads(cfg, seed, device="cpu", scale_numel=frac)
     n = sum(g.numel() for g in grads)
     ddt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[cfg.bucket_dtype]
@@ -82,34 +376,35 @@ def cpu_baseline(cfg, seed: int, budget_s: float):
         views.append(bucket.narrow(0, off, g.numel()).view(g.shape))
         off += g.numel()
     s, d = grads[0].element_size(), bucket.element_size()
-    best = float("inf")
-    t_start = time.perf_counter()
-    reps = 0
-    while reps < 5 and (reps < 2 or time.perf_counter() - t_start < budget_s):
+    oracle.reference_step_cpu(grads, views, cfg.inv_scale, cfg.max_norm)      # warm-up
+    best, reps, t_start = float("inf"), 0, time.perf_counter()
+    coef = None
+    while reps < 5 and (reps < 1 or time.perf_counter() - t_start < budget_s):
         t0 = time.perf_counter()
         ovf, norm, coef = oracle.reference_step_cpu(grads, views, cfg.inv_scale, cfg.max_norm)
-        dt = time.perf_counter() - t0
-        if reps > 0 or dt > budget_s / 2:
-            best = min(best, dt)
+        best = min(best, time.perf_counter() - t0)
         reps += 1
     nbytes = ((2 * s + d) if coef is not None else (s + d)) * n
     return {
-        "value": round(nbytes / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "value": round(nbytes / best / 1e9, 3), "unit": "GB/s", "cores": threads, "host_cpus": os.cpu_count(),
+        "kind": "port",
         "sample": f"{cfg.key}: same {len(grads)}-tensor list, {n} of {cfg.total_numel} elements "
-                  f"(dim-0 fraction {frac:.3f}), best of {max(1, reps - 1)} steps of {best * 1e3:.1f} ms, "
-                  f"torch {torch.__version__} CPU ops, {cpu_model()}",
+                  f"(dim-0 fraction {frac:.3f}), 1 warm-up + best of {reps} steps of {best * 1e3:.1f} ms, "
+                  f"torch {torch.__version__} CPU ops on {threads} threads of {os.cpu_count()} host CPUs, {cpu_model()}",
         "elements_per_s": round(n / best, 1),
     }
 
 
-def bench_optimizer(args, cfg, torch, dev) -> dict:
+# ----------------------------------------------------------------------------- optimizer step
+
+def bench_optimizer(args, key, torch, dev) -> dict:
     """Adam (+ bf16/fp16 model copy) or plain SGD over the workload's tensors: fp32 masters, fp32
     master gradients laid out as views of one packed bucket, separately allocated moments."""
     from rannc_amd import _lib
-    from rannc_amd.multi_tensor import stream_handle
-    from rannc_amd.workloads import make_grads
+    from rannc_amd.multi_tensor import TensorPlan, stream_handle
+    from rannc_amd.workloads import make_grads, step_config
 
-    from rannc_amd.multi_tensor import TensorPlan
+    cfg = step_config(key)
     grads, _ = make_grads(cfg, args.seed, device=str(dev))
     shapes = [g.shape for g in grads]
     copy_dt = grads[0].dtype if grads[0].dtype != torch.float32 else torch.bfloat16
@@ -152,28 +447,15 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
         else:
             table.sgd_step(0.01, stream=st)
 
-    for _ in range(max(0, 20 - args.warmup) + args.warmup):      # warm-up, at least 20 steps so the clocks have ramped
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()                       # the kernel is launched on torch's current stream, where these events sit
-    for _ in range(args.steps):
-        step()
-    e1.record()
-    while not e1.query():             # poll: a blocking wait adds its wake-up latency to the last step
-        pass
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    launch_ms = e0.elapsed_time(e1) / args.steps
+    step_s, launch_s = timed(step, args.steps, args.warmup, 20)
     gs = gsrc[0].element_size()
     if direct:
         bytes_per_elem = gs + (gs + 12) + 12 + 2      # read pass + Adam (grad, p, m, v in; p, m, v, copy out)
     else:
         bytes_per_elem = (16 + 12 + 2) if adam else (8 + 4 + 2)
     step_bytes = bytes_per_elem * n
-    step_s = elapsed / args.steps
-    achieved = step_bytes / (launch_ms * 1e-3) / 1e9
+    kernel = ("pass_kernel<reduce> + finalize + optim_kernel<adam>, all launches of a step" if direct
+              else f"optim_kernel<{args.op}, streaming>")
     out = {
         "metric": f"achieved HBM GB/s for the multi-tensor {args.op} step with model copy-back",
         "value": round(step_bytes / step_s / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -182,12 +464,7 @@ def bench_optimizer(args, cfg, torch, dev) -> dict:
         "config": {"workload": cfg.key, "op": args.op, "tensors": len(params), "elements": n,
                    "bytes_per_elem": bytes_per_elem, "model_copy_dtype": str(copy_dt), "seed": args.seed},
         "pct_of_hbm_peak": round(100.0 * step_bytes / step_s / 1e9 / HBM_PEAK_GBPS, 2),
-        "roofline": {"bound": "hbm", "kernel": ("pass_kernel<reduce> + finalize + optim_kernel<adam>, all launches of a step"
-                                                 if direct else f"optim_kernel<{args.op}, streaming>"),
-                     "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES_ADAM.get(cfg.key) if args.op == "adam" else None,
-                     "algorithmic_bytes_per_launch": step_bytes, "avg_launch_ms": round(launch_ms, 4)},
+        "roofline": roofline(kernel, step_bytes, launch_s, measured_traffic(args.op, cfg.key, "optim_kernel")),
     }
     table.close()
     if plan is not None:
@@ -231,9 +508,49 @@ def cpu_baseline_optimizer(op: str, shapes, seed: int, budget_s: float, bytes_pe
         reps += 1
         del copies
     return {"value": round(bytes_per_elem * total / best / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port", "cpu": cpu_model(),
+            "host_cpus": os.cpu_count(), "kind": "port", "cpu": cpu_model(),
             "sample": f"first {len(take)} tensors ({total} elements) of the workload, best of {reps} passes of "
                       f"torch.optim's per-tensor op sequence + master->bf16 copy"}
+
+
+# ----------------------------------------------------------------------------- main
+
+def headline_line(args, e: dict, w_desc: dict, dtype: str) -> dict:
+    out = {
+        "metric": "achieved HBM GB/s (% of roofline) for fused unscale+norm+clip+pack per step",
+        "value": e["GB/s"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": e["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": dict(w_desc, op=e["op"], algorithmic_bytes_per_step=e["algorithmic_bytes_per_step"], seed=args.seed,
+                       **{k: e[k] for k in ("clipped", "overflow", "skipped", "norm", "coef") if k in e}),
+        "pct_of_hbm_peak": e["pct_of_hbm_peak"],
+        "roofline": e["roofline"],
+    }
+    for k in ("elements_per_s", "bytes_moved_per_step", "GB/s_on_bytes_moved", "pct_of_hbm_peak_on_bytes_moved", "note"):
+        if k in e:
+            out[k] = e[k]
+    return out
+
+
+def run_one(args, key: str, op: str, steps: int, warmup: int) -> tuple:
+    """One (workload, operation) measurement -> (entry, workload description, dtype string)."""
+    if op in C5_OPS:
+        z = ZeroFlat(args.c5_elements, args.seed)
+        e = run_c5(z, op, steps, warmup)
+        z.close()
+        return e, {"workload": "c5_zero_flat", "description": "ZeRO flat fp16 buffer, 4096 odd-sized segments at odd offsets",
+                   "elements": e["elements"]}, "f16 / f32 copies"
+    w = StepWorkload(key, args.seed, args.chunk_elems)
+    if op in ("fused_step", "fused_step_noclip", "fused_step_noclip_2pass"):
+        e = run_fused_step(w, steps, warmup, op)
+    elif op == "overflow_host_gate":
+        e = run_overflow_host_gate(w, steps, warmup)
+    else:
+        e = run_plan_op(w, op, steps, warmup)
+    desc = w.describe()
+    dtype = f"{w.cfg.grad_dtype}->{w.cfg.bucket_dtype} (fp32 arithmetic)"
+    w.close()
+    return e, desc, dtype
 
 
 def main() -> int:
@@ -245,18 +562,11 @@ def main() -> int:
         return 2
 
     import torch
-    from rannc_amd.multi_tensor import TensorPlan
-    from rannc_amd.workloads import make_grads, step_config
-
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    cfg = step_config(args.workload)
-    if args.op != "fused_step":
-        print(json.dumps(bench_optimizer(args, cfg, torch, dev)), flush=True)
-        return 0
     if args.calibrate_copy:
         a = torch.empty(256 << 20, dtype=torch.float32, device=dev).fill_(1.0)
         b = torch.empty_like(a)
@@ -265,96 +575,57 @@ def main() -> int:
         torch.cuda.synchronize()
         del a, b
         torch.cuda.empty_cache()
-    grads, _ = make_grads(cfg, args.seed, device=str(dev))
-    n = sum(g.numel() for g in grads)
-    ddt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[cfg.bucket_dtype]
-    bucket = torch.zeros(n, dtype=ddt, device=dev)
-    dsts, off = [], 0
-    for g in grads:
-        dsts.append(bucket.narrow(0, off, g.numel()))
-        off += g.numel()
-    s, d = grads[0].element_size(), bucket.element_size()
 
-    plan = TensorPlan(grads, dsts, chunk_elems=args.chunk_elems)
-    # Untimed: the W warm-up steps asked for, preceded by enough further steps (about 25 ms of work)
-    # that the GPU has left its idle clocks before anything is timed.
-    for _ in range(max(0, 60 - args.warmup) + args.warmup):
-        plan.fused_step(cfg.inv_scale, cfg.max_norm)
-    torch.cuda.synchronize()
-    # Timed region: HIP events (recorded by the library on the launch stream) bracket only the
-    # dominant kernel, the write pass, and only on every fifth step: each record costs a few
-    # microseconds of stream time, which would otherwise be part of every step measured here.
-    stride = min(5, max(1, args.steps))
-    sampled = (args.steps + stride - 1) // stride
-    plan.plan.enable_timing(-sampled)
-    plan.plan.timing_stride(stride)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        plan.fused_step(cfg.inv_scale, cfg.max_norm)
-    done = torch.cuda.Event()
-    done.record()
-    while not done.query():       # poll: a blocking wait adds its wake-up latency to the last step
-        pass
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    res = plan.result()
-    write_only = [plan.plan.read_timing(i) for i in range(sampled)]
-    plan.plan.timing_stride(1)
-    # A second, untimed loop brackets all three stages for the breakdown.
-    plan.plan.enable_timing(args.steps)
-    for _ in range(args.steps):
-        plan.fused_step(cfg.inv_scale, cfg.max_norm)
-    torch.cuda.synchronize()
-    per_kernel = [plan.plan.read_timing(i) for i in range(args.steps)]
-    plan.plan.enable_timing(0)
+    everything = args.op in (None, "all") and args.workload is None
+    if args.op in OPTIM_OPS:
+        print(json.dumps(bench_optimizer(args, args.workload or "c2_bert_large", torch, dev)), flush=True)
+        return 0
 
-    step_s = elapsed / args.steps
-    clipped = bool(res.clipped)
-    step_bytes = ((2 * s + d) if clipped else (s + d)) * n
-    value = step_bytes / step_s / 1e9
+    key = args.workload or HEADLINE
+    op = args.op if args.op not in (None, "all") else ("c5_unflatten" if key == "c5_zero_flat" else "fused_step")
+    e, desc, dtype = run_one(args, key, op, args.steps, args.warmup)
+    out = headline_line(args, e, desc, dtype)
 
-    # dominant kernel: the write pass (re-read s*N, write d*N)
-    write_ms = sum(k[2] for k in write_only) / len(write_only)
-    reduce_ms = sum(k[0] for k in per_kernel) / len(per_kernel)
-    final_ms = sum(k[1] for k in per_kernel) / len(per_kernel)
-    write_bytes = (s + d) * n
-    achieved = write_bytes / (write_ms * 1e-3) / 1e9
-    roofline = {
-        "bound": "hbm", "kernel": "pass_kernel<write, streaming>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.key),
-        "algorithmic_bytes_per_launch": write_bytes, "avg_launch_ms": round(write_ms, 4),
-        "launches_timed": len(write_only),
-        "other_kernels": {
-            "pass_kernel<reduce>": {"avg_launch_ms": round(reduce_ms, 4), "algorithmic_bytes_per_launch": s * n,
-                                    "achieved": round(s * n / (reduce_ms * 1e-3) / 1e9, 1)},
-            "finalize_tensors_kernel+finalize_total_kernel": {"avg_launch_ms": round(final_ms, 4)},
-            "note": "from a second, untimed loop of the same steps with all stages bracketed",
-        },
-    }
+    if everything:
+        # every other configuration and operation of the path, each measured like the headline (their own step
+        # counts: sub-millisecond steps need more of them for the first launch not to weigh)
+        sub = max(args.steps, 50)
+        plan = [
+            ("c3_bert_enlarged_overflow", "fused_step", args.steps), ("c3_bert_enlarged_overflow", "overflow_host_gate", args.steps),
+            ("c3_bert_enlarged", "fused_step_noclip", args.steps), ("c3_bert_enlarged", "unscale_pack", args.steps),
+            ("c2_bert_large", "fused_step", sub), ("c2_bert_large", "fused_step_noclip", sub),
+            ("c2_bert_large", "fused_step_noclip_2pass", sub), ("c2_bert_large", "unscale_pack", sub),
+            ("c2_bert_large", "copy_back", sub),
+            ("c4_resnet152x2", "fused_step", sub), ("c4_resnet152x2", "fused_step_noclip", sub),
+            ("c1_mlp", "fused_step", 4 * sub), ("c1_mlp", "unflatten_back", 4 * sub),
+        ]
+        configs = []
+        cur_key, w = None, None
+        for k2, op2, st in plan:
+            if k2 != cur_key:
+                if w is not None:
+                    w.close()
+                w, cur_key = StepWorkload(k2, args.seed, args.chunk_elems), k2
+            if op2 in ("fused_step", "fused_step_noclip", "fused_step_noclip_2pass"):
+                configs.append(run_fused_step(w, st, args.warmup, op2))
+            elif op2 == "overflow_host_gate":
+                configs.append(run_overflow_host_gate(w, st, args.warmup))
+            else:
+                configs.append(run_plan_op(w, op2, st, args.warmup))
+        if w is not None:
+            w.close()
+        free, _ = torch.cuda.mem_get_info()
+        if args.c5_elements * 8 < free * 0.9:
+            z = ZeroFlat(args.c5_elements, args.seed)
+            for op5 in C5_OPS:
+                configs.append(run_c5(z, op5, max(5, min(args.steps, 10)), 2))
+            z.close()
+        else:
+            configs.append({"workload": "c5_zero_flat", "skipped": f"needs {args.c5_elements * 8 / 1e9:.0f} GB of device memory"})
+        out["configs"] = configs
 
-    out = {
-        "metric": "achieved HBM GB/s (% of roofline) for fused unscale+norm+clip+pack per step",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": f"{cfg.grad_dtype}->{cfg.bucket_dtype} (fp32 arithmetic)",
-        "data": "synthetic",
-        "config": {"workload": cfg.key, "description": cfg.description, "tensors": len(grads), "elements": n,
-                   "src_bytes_per_elem": s, "dst_bytes_per_elem": d,
-                   "algorithmic_bytes_per_step": step_bytes, "clipped": clipped, "overflow": int(res.overflow),
-                   "norm": res.norm, "coef": res.coef, "seed": args.seed,
-                   "chunk_elems": plan.plan.chunk_elems, "chunks": plan.plan.num_chunks,
-                   "untimed_steps_before_timing": max(0, 60 - args.warmup) + args.warmup},
-        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
-        "elements_per_s": round(n / step_s, 1),
-        "roofline": roofline,
-    }
-    plan.close()
-    del grads, bucket, dsts
-    torch.cuda.empty_cache()
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, args.seed, args.cpu_seconds)
+    if not args.no_cpu_baseline and key != "c5_zero_flat":
+        out["cpu_baseline"] = cpu_baseline(key, args.seed, args.cpu_seconds)
     print(json.dumps(out), flush=True)
     return 0
 

@@ -53,7 +53,18 @@ enum {
   /* Report the flag but let it gate nothing: a non-finite norm then behaves exactly as in
    * ParamStorage::clipGradNorm (inf -> coef 0, NaN -> no clip; src/comp/ParamStorage.cpp:723-742).
    * This is what RaNNCModule.clip_grad_norm on existing gradients uses. */
-  RG_STEP_IGNORE_OVERFLOW = 2
+  RG_STEP_IGNORE_OVERFLOW = 2,
+  /* The caller expects that this step will not clip (its last one did not).  The step then
+   * runs as ONE pass that writes the unscaled values while it sums them - (s + d) bytes per
+   * element instead of (2s + d) - followed by the decision; only if the decision is "clip"
+   * after all does a second kernel multiply the destination in place by the coefficient
+   * ((s + 3d) bytes in that case).  Norm, flag, coefficient and every written bit are those
+   * of the default strategy (the norm to rounding: its partial sums are taken per tile); on
+   * overflow the destination holds the unscaled values (as with RG_STEP_WRITE_ON_OVERFLOW).
+   * In place with inv_scale == 1 (clip_grad_norm on existing gradients) a step that does not
+   * clip writes nothing under either strategy; the flag then only makes the gated second
+   * kernel cheaper to find idle. */
+  RG_STEP_EXPECT_NO_CLIP = 4
 };
 
 const char* rg_last_error(void);

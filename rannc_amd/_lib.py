@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("RANNC_AMD_LIB") or os.path.join(HERE, "libranncgrad.s
 
 RG_OK, RG_EINVAL, RG_EALIGN, RG_EHIP, RG_ENOMEM = 0, 1, 2, 3, 4
 RG_F32, RG_F16, RG_BF16 = 0, 1, 2
-RG_STEP_DEFAULT, RG_STEP_WRITE_ON_OVERFLOW, RG_STEP_IGNORE_OVERFLOW = 0, 1, 2
+RG_STEP_DEFAULT, RG_STEP_WRITE_ON_OVERFLOW, RG_STEP_IGNORE_OVERFLOW, RG_STEP_EXPECT_NO_CLIP = 0, 1, 2, 4
 
 DTYPE_CODES = {"f32": RG_F32, "f16": RG_F16, "bf16": RG_BF16}
 

@@ -46,6 +46,7 @@ struct rg_plan {
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
   bool dst_heads = false;            // some destination starts off a 128-byte boundary
   bool offgrid = false;              // some source is off the 128-byte grid of its destination
+  bool all_in_place = false;         // every tensor with elements has dst == src (and so one dtype)
 
   // one device allocation, carved up
   char* dev_base = nullptr;
@@ -94,8 +95,10 @@ static int64_t tensor_head(const void* src, const void* dst, int ss, int ds) {
 static void fill_chunk_records(rg_plan* p, ChunkRec* out) {
   p->dst_heads = false;
   p->offgrid = false;
+  p->all_in_place = true;
   for (int i = 0; i < p->n_tensors; ++i) {
     const TensorDesc& t = p->host_tensors[(size_t)i];
+    if (t.numel > 0 && (t.dst == nullptr || t.dst != t.src)) p->all_in_place = false;
     const int ss = elem_size(t.src_dtype), ds = elem_size(t.dst_dtype);
     const int64_t head = tensor_head(t.src, t.dst, ss, ds);
     if (t.dst != nullptr && t.numel > 0 && head != 0) p->dst_heads = true;
@@ -234,15 +237,17 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   // The Infinity Cache holds 256 MiB: below that a second pass can still hit in cache.
   p->streaming = bytes > (int64_t)256 << 20;
   p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total);
-  // Tuning knobs, read once per plan (defaults are what measured best on MI355X):
+  // Tuning knobs of experiment builds, read once per plan (defaults are what measured best on MI355X):
   //   RG_WRITE_TILE_ELEMS    elements per block of a writing pass (>= 256)
   //   RG_XCD_REDUCE / _WRITE block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run);
   //                          unset, writing passes use 0, or runs of 256 when a source is off its destination's line grid
   //   RG_REDUCE_TILE_FACTOR  tile of a reducing + writing pass, in write tiles (0 = per operation)
+#ifdef RG_TUNING_ENV   // experiment builds only: the shipped library takes no launch shape from the environment
   if (const char* env = getenv("RG_WRITE_TILE_ELEMS")) p->write_tile_elems = atoll(env);
   if (const char* env = getenv("RG_XCD_REDUCE")) p->xcd_reduce = atoi(env);
   if (const char* env = getenv("RG_XCD_WRITE")) p->xcd_write = p->xcd_write_offgrid = atoi(env);
   if (const char* env = getenv("RG_REDUCE_TILE_FACTOR")) p->reduce_tile_factor = atoll(env);
+#endif
   if (p->reduce_tile_factor < 0) p->reduce_tile_factor = 0;
 
   p->chunk_begin.assign((size_t)n + 1, 0);
@@ -270,7 +275,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   const size_t max_tiles = (size_t)((p->chunk_elems + p->write_tile_elems - 1) / p->write_tile_elems);
   const size_t o_sumsq = carve(nc * sizeof(double));
   const size_t o_bad = carve(nc * sizeof(int32_t));
-  const size_t tile_partials = nc * max_tiles;
+  const size_t tile_partials = nc * max_tiles * (size_t)(kWriteThreads / 64);   // one per wavefront of every tile
   const size_t o_tile_sumsq = carve(tile_partials * sizeof(double));
   const size_t o_tile_bad = carve(tile_partials * sizeof(int32_t));
   const size_t o_tnorm = carve(nt * sizeof(float));
@@ -432,25 +437,31 @@ static void split_for_write(const rg_plan* p, PassArgs& a) {
   }
 }
 
-// One pass that both reduces and writes, over tiles of each chunk: every tile leaves its own
-// partial sum, and the per-tensor finalize adds the tile partials directly.
-static int tiled_reduce_write(rg_plan* p, PassArgs& a, int mode, hipStream_t s) {
+// One pass that both reduces and writes, over tiles of each chunk: every wavefront of every
+// tile leaves its own partial sum; a small kernel folds them into per-chunk sums, which the
+// per-tensor finalize then adds as it does after a read-only pass.
+static int tiled_reduce_write(rg_plan* p, PassArgs& a, int mode, hipStream_t s, float max_norm = 0.0f,
+                              int ignore_overflow = 0, hipEvent_t after_pass = nullptr) {
   split_for_write(p, a);
-  // measured on MI355X: twice the write tile is best for unscale+pack, the plain write tile when accumulating
-  const int64_t factor = p->reduce_tile_factor > 0 ? p->reduce_tile_factor : ((mode & kModeAccumulate) ? 1 : 2);
+  // measured on MI355X: the plain write tile is best now that no block-wide combine ends a tile
+  const int64_t factor = p->reduce_tile_factor > 0 ? p->reduce_tile_factor : 1;
   if (a.tiles_per_chunk > 1 && factor > 1 && a.tile_elems * factor <= p->chunk_elems) {
-    // every tile of this pass also pays a block-wide reduction: a larger tile amortises it
     a.tile_elems = (int32_t)(a.tile_elems * factor);
     a.tiles_per_chunk = (int32_t)((p->chunk_elems + a.tile_elems - 1) / a.tile_elems);
   }
-  FinalizeArgs f = finalize_args(p, 0.0f, 0);
   a.chunk_sumsq = p->d_tile_sumsq;
   a.chunk_bad = p->d_tile_bad;
-  f.chunk_sumsq = p->d_tile_sumsq;
-  f.chunk_bad = p->d_tile_bad;
-  f.partials_per_chunk = a.tiles_per_chunk;
   RG_HIP(launch_pass(mode, a, p->streaming, s));
-  RG_HIP(launch_finalize(f, s));
+  if (after_pass) RG_HIP(hipEventRecord(after_pass, s));
+  CombineArgs c;
+  c.tile_sumsq = p->d_tile_sumsq;
+  c.tile_bad = p->d_tile_bad;
+  c.chunk_sumsq = p->d_chunk_sumsq;
+  c.chunk_bad = p->d_chunk_bad;
+  c.n_chunks = p->n_chunks;
+  c.partials_per_chunk = a.tiles_per_chunk * (kWriteThreads / 64);
+  RG_HIP(launch_combine_tiles(c, s));
+  RG_HIP(launch_finalize(finalize_args(p, max_norm, ignore_overflow), s));
   return RG_OK;
 }
 
@@ -491,6 +502,26 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
     ev = &p->timing_events[(size_t)(p->timing_count++ % p->timing_slots) * 4];
   PassArgs a = pass_args(p, inv_scale);
   const bool all = ev != nullptr && p->timing_all;
+  // In place with inv_scale == 1 a step that does not clip leaves every value as it is: the
+  // second pass then has nothing to write and is gated on the decision.
+  const bool identity_unless_clipped = p->all_in_place && inv_scale == 1.0f;
+  if ((flags & RG_STEP_EXPECT_NO_CLIP) && !identity_unless_clipped) {
+    // One pass writes the unscaled values while it sums them; only if the decision then says
+    // "clip" does a second kernel scale the destination in place.  That kernel's blocks cover
+    // whole chunks, so finding that there is nothing to do costs a few microseconds.
+    if (all) RG_HIP(hipEventRecord(ev[0], s));
+    const int rc1 = tiled_reduce_write(p, a, kModeReduce | kModeWrite, s, max_norm,
+                                       (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0, all ? ev[1] : nullptr);
+    if (rc1 != RG_OK) return rc1;
+    if (ev) RG_HIP(hipEventRecord(ev[2], s));
+    PassArgs b = pass_args(p, 1.0f);
+    b.result = p->d_result;
+    b.only_if_clipped = 1;
+    b.src_is_dst = 1;
+    RG_HIP(launch_pass(kModeWrite, b, p->streaming, s));
+    if (ev) RG_HIP(hipEventRecord(ev[3], s));
+    return RG_OK;
+  }
   if (all) RG_HIP(hipEventRecord(ev[0], s));
   a.xcd_run = p->xcd_reduce;
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
@@ -499,8 +530,10 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
+  a.only_if_clipped = identity_unless_clipped ? 1 : 0;
   a.xcd_run = p->offgrid ? p->xcd_write_offgrid : p->xcd_write;
-  split_for_write(p, a);
+  // a launch that will most likely find nothing to do keeps one block per chunk: fewer blocks to retire
+  if (!(identity_unless_clipped && (flags & RG_STEP_EXPECT_NO_CLIP))) split_for_write(p, a);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, s));
   if (ev) RG_HIP(hipEventRecord(ev[3], s));
   return RG_OK;

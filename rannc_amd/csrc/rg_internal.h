@@ -115,6 +115,8 @@ struct PassArgs {
   int32_t write_on_overflow;
   int32_t zero_fill;             // write pass: ignore the sources, store zeros
   int32_t norm_of_source;        // reduce pass: measure the source as stored (no rounding to dst)
+  int32_t only_if_clipped;       // with `result`: the whole launch does nothing unless result->clipped is set
+  int32_t src_is_dst;            // read the destination instead of the record's source (in-place rescale)
 };
 
 struct FinalizeArgs {
@@ -133,10 +135,20 @@ struct FinalizeArgs {
   int32_t partials_per_chunk;  // 1, or the tiles per chunk of a tiled reducing pass
 };
 
+struct CombineArgs {
+  const double* tile_sumsq;   // [n_chunks * partials_per_chunk], chunk-major
+  const int32_t* tile_bad;
+  double* chunk_sumsq;        // [n_chunks]
+  int32_t* chunk_bad;
+  int64_t n_chunks;
+  int32_t partials_per_chunk;
+};
+
 // streaming: nontemporal loads/stores (data far larger than the caches).
 hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream);
 hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream);
+hipError_t launch_combine_tiles(const CombineArgs& a, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
 
 void set_error(const char* fmt, ...);

@@ -220,7 +220,11 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
   float coef = 1.0f;
   if (a.result != nullptr) {
     // Values produced by the finalize kernel earlier on the same stream.
-    if (a.result->skipped != 0 && a.write_on_overflow == 0) return;
+    if (a.only_if_clipped != 0) {
+      if (a.result->clipped == 0) return;
+    } else if (a.result->skipped != 0 && a.write_on_overflow == 0) {
+      return;
+    }
     coef = a.result->coef;
   }
 
@@ -248,14 +252,22 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
   const int start = tile == 0 ? 0 : chunk_head + tile * a.tile_elems;
   int end = tile == a.tiles_per_chunk - 1 ? rec.len : chunk_head + (tile + 1) * a.tile_elems;
   if (end > rec.len) end = rec.len;
+  // A pass that reduces and writes leaves one partial per wavefront (no block-wide combine at
+  // the end of a tile that only lives a few microseconds); a read-only pass one per block.
+  constexpr bool kWavePartials = (MODE & kModeReduce) != 0 && (MODE & kModeWrite) != 0;
+  constexpr int kSlots = kWavePartials ? T / 64 : 1;
   if (start >= end) {
-    if ((MODE & kModeReduce) && threadIdx.x == 0) {
-      a.chunk_sumsq[bid] = 0.0;
-      a.chunk_bad[bid] = 0;
+    if ((MODE & kModeReduce) && threadIdx.x < kSlots) {
+      a.chunk_sumsq[(size_t)bid * kSlots + threadIdx.x] = 0.0;
+      a.chunk_bad[(size_t)bid * kSlots + threadIdx.x] = 0;
     }
     return;
   }
   const int len = end - start;
+  if (a.src_is_dst) {
+    rec.src = rec.dst;
+    rec.src_dtype = rec.dst_dtype;
+  }
   const char* sp = rec.src ? reinterpret_cast<const char*>(rec.src) + (size_t)start * (rec.src_dtype == RG_F32 ? 4 : 2) : nullptr;
   char* dp = reinterpret_cast<char*>(rec.dst) + (size_t)start * (rec.dst_dtype == RG_F32 ? 4 : 2);
   const int src_kind = rec.src_dtype;
@@ -312,7 +324,28 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
     double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
                (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
     s = wave_total(s);
-    {
+    if constexpr (kWavePartials) {
+      // One partial per wavefront.  A wavefront whose sum is not finite looks at every element
+      // of the tile again (its own elements are strided through it), 64 at a time.
+      int bad = 0;
+      if (!(fabs(s) <= 1.79769313486231570e308)) {
+        int mine = 0;
+        if (sp != nullptr) {
+          const int lane = threadIdx.x & 63;
+          const int es = src_kind == RG_F32 ? 4 : 2;
+          for (int i = lane; i < len; i += 64) {
+            const char* q = sp + (size_t)i * es;
+            mine |= (src_kind == RG_F32 ? nonfinite_at<RG_F32>(q) : src_kind == RG_F16 ? nonfinite_at<RG_F16>(q)
+                                                                                        : nonfinite_at<RG_BF16>(q)) ? 1 : 0;
+          }
+        }
+        bad = __any(mine) ? 1 : 0;
+      }
+      if ((threadIdx.x & 63) == 0) {
+        a.chunk_sumsq[(size_t)bid * kSlots + (threadIdx.x >> 6)] = s;
+        a.chunk_bad[(size_t)bid * kSlots + (threadIdx.x >> 6)] = bad;
+      }
+    } else {
       // One partial per block, the wavefronts combined through LDS in index order.
       __shared__ double wave_sum[kWaves];
       if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = s;
@@ -351,6 +384,30 @@ __device__ __forceinline__ void block_sum_or(double& s, int& bad, double* lds_su
   s = (lds_sum[0] + lds_sum[1]) + (lds_sum[2] + lds_sum[3]);
   bad = lds_bad[0] | lds_bad[1] | lds_bad[2] | lds_bad[3];
   __syncthreads();
+}
+
+// After a pass that left one partial per wavefront of every tile: wavefront w of the grid adds
+// the partials of chunk w in a fixed order into the chunk's slot of the per-chunk arrays, so
+// that the per-tensor kernel below sees the same number of values whatever pass produced them
+// (a large tensor has tens of thousands of tile partials, too many for its one block).
+__global__ __launch_bounds__(kBlockThreads) void combine_tiles_kernel(CombineArgs a) {
+  const int64_t c = (int64_t)blockIdx.x * (kBlockThreads / 64) + (threadIdx.x >> 6);
+  if (c >= a.n_chunks) return;
+  const int lane = threadIdx.x & 63;
+  const double* ps = a.tile_sumsq + c * a.partials_per_chunk;
+  const int32_t* pb = a.tile_bad + c * a.partials_per_chunk;
+  double s = 0.0;
+  int bad = 0;
+  for (int i = lane; i < a.partials_per_chunk; i += 64) {
+    s += ps[i];
+    bad |= pb[i];
+  }
+  s = wave_total(s);
+  bad = __any(bad) ? 1 : 0;
+  if (lane == 0) {
+    a.chunk_sumsq[c] = s;
+    a.chunk_bad[c] = bad;
+  }
 }
 
 // Block t reduces tensor t's chunk sums (thread-strided with four independent loads in
@@ -478,6 +535,14 @@ hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream) {
   if (a.n_tensors > 0)
     hipLaunchKernelGGL(finalize_tensors_kernel, dim3((unsigned)a.n_tensors), dim3(kBlockThreads), 0, stream, a);
   hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine_tiles(const CombineArgs& a, hipStream_t stream) {
+  if (a.n_chunks <= 0) return hipSuccess;
+  const int per_block = kBlockThreads / 64;
+  hipLaunchKernelGGL(combine_tiles_kernel, dim3((unsigned)((a.n_chunks + per_block - 1) / per_block)), dim3(kBlockThreads), 0,
+                     stream, a);
   return hipGetLastError();
 }
 
