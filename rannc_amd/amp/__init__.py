@@ -52,7 +52,8 @@ class _AmpStash:
         self.already_patched = False
         self.lazy_init_called = False
         self.unscale_plan: Optional[TensorPlan] = None
-        self.unscale_key: Optional[tuple] = None
+        self.unscale_cache = None          # param_storage._PlanCache holding unscale_plan
+        self.step_flags = _lib.RG_STEP_DEFAULT      # RG_STEP_IGNORE_OVERFLOW under a static loss scale
         self.copy_back_plan: Optional[TensorPlan] = None
         self.pending_finish = False        # fused mode: the write pass has not run yet
         self.pending_inv_scale = 1.0       #   ... the 1/loss_scale its read pass ran with
@@ -99,12 +100,12 @@ class LossScaler:
         inf/NaN flag and - for free - the gradient norm.  In fused mode only the read pass runs
         here; the values are written by ``finish_unscale``.  ``accumulate`` adds to the master
         gradients instead of overwriting them (always eager)."""
-        key = tuple((g.data_ptr(), g.numel(), g.dtype, m.data_ptr(), m.dtype) for g, m in zip(model_grads, master_grads))
-        if stash.unscale_plan is None or stash.unscale_key != key:
-            if stash.unscale_plan is not None:
-                stash.unscale_plan.close()
-            stash.unscale_plan = TensorPlan(model_grads, master_grads)
-            stash.unscale_key = key
+        # One device table for the whole run: when backward hands back gradients at new addresses (same
+        # sizes and dtypes) the table is re-pointed in place, stream ordered - nothing is freed or allocated.
+        if stash.unscale_cache is None:
+            from ..param_storage import _PlanCache
+            stash.unscale_cache = _PlanCache()
+        stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads)
         inv = 1.0 / self._loss_scale
         with torch.no_grad():
             if accumulate:
@@ -119,6 +120,11 @@ class LossScaler:
         stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
         if stash.last_result.overflow:
             self._has_overflow = True
+        if not stash.pending_finish:
+            # every kernel that reads the model gradients is queued: let go of them, so that backward
+            # finds their memory free again (and, in the steady state, at the same addresses)
+            stash.unscale_plan.drop_sources()
+            stash.pending_model_grads = []
 
     def update_scale(self) -> bool:
         """Returns True when the step must be skipped.  Own schedule (see module docstring)."""
@@ -171,6 +177,11 @@ def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_lev
     stash.fused = fused
     optimizer._amp_stash = stash
     scaler = LossScaler(loss_scale, min_loss_scale=min_loss_scale, max_loss_scale=max_loss_scale)
+    # A static scale never skips a step (Apex): an overflow must then reach the master gradients and the
+    # optimizer as the inf/NaN it is - in fused mode too - instead of leaving last step's values in place.
+    # RG_STEP_IGNORE_OVERFLOW makes the deferred write / the clip decision behave exactly like
+    # ParamStorage::clipGradNorm on gradients that contain them (src/comp/ParamStorage.cpp:723-742).
+    stash.step_flags = _lib.RG_STEP_DEFAULT if scaler.dynamic else _lib.RG_STEP_IGNORE_OVERFLOW
     _amp_state.loss_scalers = [scaler]
     _amp_state.opt_level = opt_level
     _patch_step(optimizer)
@@ -221,9 +232,11 @@ def finish_unscale(optimizer: torch.optim.Optimizer, max_norm: Optional[float] =
         if max_norm is None:
             max_norm = stash.decided_max_norm or 0.0
         with torch.no_grad():
-            stash.unscale_plan.step_finish(float(max_norm))
+            stash.unscale_plan.step_finish(float(max_norm), stash.step_flags)
         stash.pending_finish = False
         stash.decided_max_norm = None
+        stash.unscale_plan.drop_sources()
+        stash.pending_model_grads = []
 
 
 def can_step_from_model_grads(optimizer: torch.optim.Optimizer) -> bool:
@@ -241,7 +254,7 @@ def decide_clip(optimizer: torch.optim.Optimizer, max_norm: float) -> None:
     gradients); the optimizer's step kernel applies it while reading the model gradients."""
     stash = optimizer._amp_stash
     with torch.no_grad():
-        stash.unscale_plan.step_decide(float(max_norm))
+        stash.unscale_plan.step_decide(float(max_norm), stash.step_flags)
     stash.decided_max_norm = float(max_norm)
 
 
@@ -268,6 +281,9 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
         if getattr(stash, "skip_next_step", False):
             stash.skip_next_step = False
             stash.pending_finish = False
+            if stash.unscale_plan is not None:
+                stash.unscale_plan.drop_sources()
+            stash.pending_model_grads = []
             return None
         if can_step_from_model_grads(optimizer) and not (args or kwargs):
             # unscale, clip, update and model copy in one kernel: the step reads the still-scaled
@@ -284,6 +300,8 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
                 optimizer.grad_scale, optimizer.gate = 1.0, 0
             stash.pending_finish = False
             stash.decided_max_norm = None
+            stash.unscale_plan.drop_sources()
+            stash.pending_model_grads = []
             return ret
         finish_unscale(optimizer)
         ret = old_step(*args, **kwargs)

@@ -249,6 +249,7 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
     chunk_head = head_elems(reinterpret_cast<uintptr_t>(rec.dst), kWriteAlignBytes, rec.dst_dtype == RG_F32 ? 4u : 2u);
     if (chunk_head > rec.len) chunk_head = rec.len;
   }
+  const size_t slot_id = bid;   // of this block's partial sums
   const int start = tile == 0 ? 0 : chunk_head + tile * a.tile_elems;
   int end = tile == a.tiles_per_chunk - 1 ? rec.len : chunk_head + (tile + 1) * a.tile_elems;
   if (end > rec.len) end = rec.len;
@@ -258,8 +259,8 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
   constexpr int kSlots = kWavePartials ? T / 64 : 1;
   if (start >= end) {
     if ((MODE & kModeReduce) && threadIdx.x < kSlots) {
-      a.chunk_sumsq[(size_t)bid * kSlots + threadIdx.x] = 0.0;
-      a.chunk_bad[(size_t)bid * kSlots + threadIdx.x] = 0;
+      a.chunk_sumsq[slot_id * kSlots + threadIdx.x] = 0.0;
+      a.chunk_bad[slot_id * kSlots + threadIdx.x] = 0;
     }
     return;
   }
@@ -342,8 +343,8 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
         bad = __any(mine) ? 1 : 0;
       }
       if ((threadIdx.x & 63) == 0) {
-        a.chunk_sumsq[(size_t)bid * kSlots + (threadIdx.x >> 6)] = s;
-        a.chunk_bad[(size_t)bid * kSlots + (threadIdx.x >> 6)] = bad;
+        a.chunk_sumsq[slot_id * kSlots + (threadIdx.x >> 6)] = s;
+        a.chunk_bad[slot_id * kSlots + (threadIdx.x >> 6)] = bad;
       }
     } else {
       // One partial per block, the wavefronts combined through LDS in index order.
@@ -364,8 +365,8 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
         bad = __syncthreads_or(mine);
       }
       if (threadIdx.x == 0) {
-        a.chunk_sumsq[bid] = total;
-        a.chunk_bad[bid] = bad;
+        a.chunk_sumsq[slot_id] = total;
+        a.chunk_bad[slot_id] = bad;
       }
     }
   }

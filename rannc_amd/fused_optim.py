@@ -26,7 +26,10 @@ class _FusedBase(torch.optim.Optimizer):
         self._model_copies: Dict[int, torch.Tensor] = {}
         self._steps: Dict[int, Tuple[torch.Tensor, int]] = {}     # id(param) -> (its step tensor, value)
         #: device pointer of an ``rg_step_result`` (``TensorPlan.plan.result_device_ptr()``): the step
-        #: multiplies the gradients by its clip coefficient and does nothing when it says "skipped"
+        #: multiplies the gradients by its clip coefficient and does nothing when it says "skipped".
+        #: The host-side bookkeeping (step counts, the first-step flag of momentum buffers) advances
+        #: regardless, so a caller that sets ``gate`` must itself skip ``step()`` whenever the device
+        #: would (``amp`` does: a dynamic scaler skips on the host, a static one never gates).
         self.gate: int = 0
         #: every gradient is multiplied by this first
         self.grad_scale: float = 1.0
@@ -183,7 +186,9 @@ class FusedSGD(_FusedBase):
                 grad_of[id(p)] = g
                 st = self.state[p]
                 if group["momentum"] != 0 and st.get("momentum_buffer") is None:
-                    st["momentum_buffer"] = torch.empty_like(p, memory_format=torch.preserve_format)
+                    # zeros, not empty: if the first launch is gated off on the device the buffer must
+                    # not reach the next step with whatever the memory held
+                    st["momentum_buffer"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                     fresh.append(p)
                 else:
                     seasoned.append(p)

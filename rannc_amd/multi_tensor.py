@@ -119,6 +119,12 @@ class TensorPlan:
         if dsts is not None:
             self._dsts = list(dsts)
 
+    def drop_sources(self) -> None:
+        """Stop keeping the source tensors alive (the table still points at their memory).  For callers
+        that have queued every kernel reading them and will ``update`` the table before its next use;
+        memory PyTorch then reuses on the same stream is ordered behind those kernels."""
+        self._srcs = [None] * len(self._srcs)
+
     def fused_step(self, inv_scale: float, max_norm: float, flags: int = _lib.RG_STEP_DEFAULT) -> None:
         self.plan.fused_step(inv_scale, max_norm, flags, self._stream())
 

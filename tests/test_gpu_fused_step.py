@@ -236,3 +236,64 @@ def test_tuning_knobs_do_not_change_results(env, monkeypatch):
     assert math.isclose(plan.result().norm, rp.result().norm, rel_tol=1e-12)
     for a, b in zip(out, ref_pack):
         assert_bits_equal(a.cpu(), b.cpu(), f"unscale_pack with {env}")
+
+
+# ----------------------------------------------------------------------------- one-pass strategy
+
+@pytest.mark.parametrize("src_name,dst_name", [("bf16", "f32"), ("f16", "f32"), ("f32", "f32"), ("f16", "f16"), ("f32", "bf16")])
+@pytest.mark.parametrize("max_norm", [0.5, 1e9])
+def test_expect_no_clip_strategy_matches_the_oracle(src_name, dst_name, max_norm):
+    """RG_STEP_EXPECT_NO_CLIP: one writing pass plus, only when the step clips after all, an in-place
+    scale - same flag, norm (1e-6), decision and written bits as the oracle, whether or not it clips."""
+    scale = 1.0 if src_name == "f32" else 256.0
+    shapes = SHAPES_SMALL + [(300001,), (70000,)]
+    grads = _grads(shapes, TORCH_DTYPE[src_name], 1e-1, scale, seed=21)
+    for lead, gap, dst_lead in ((0, 0, 0), (1, 1, 3)):
+        res, tn, out = _run_fused(grads, TORCH_DTYPE[dst_name], 1.0 / scale, max_norm, flags=_lib.RG_STEP_EXPECT_NO_CLIP,
+                                  lead=lead, gap=gap, dst_lead=dst_lead)
+        _check_against_oracle(grads, dst_name, 1.0 / scale, max_norm, res, tn, out)
+        assert res.clipped == (1 if max_norm == 0.5 else 0)
+
+
+def test_expect_no_clip_on_overflow_leaves_the_unscaled_values():
+    grads = _grads([(5000,), (17,), (40000,)], torch.float16, 1e-2, 64.0, seed=22)
+    grads[2].view(-1)[12345] = float("inf")
+    res, tn, out = _run_fused(grads, torch.float32, 1 / 64.0, 0.5, flags=_lib.RG_STEP_EXPECT_NO_CLIP)
+    assert res.overflow == 1 and res.skipped == 1 and res.clipped == 0 and res.coef == 1.0
+    want, flag = oracle.unscale_and_check(grads, 1 / 64.0)        # written as Apex's multi_tensor_scale writes them
+    assert flag == 1
+    assert_bits_equal(out, torch.cat([w.flatten() for w in want]), "unscaled values on overflow")
+
+
+@pytest.mark.parametrize("flags", [_lib.RG_STEP_IGNORE_OVERFLOW, _lib.RG_STEP_IGNORE_OVERFLOW | _lib.RG_STEP_EXPECT_NO_CLIP])
+@pytest.mark.parametrize("max_norm", [0.25, 1e9])
+def test_in_place_clip_writes_only_when_it_clips(flags, max_norm):
+    """clip_grad_norm on existing gradients (dst == src, inv_scale == 1): bits as the oracle's in-place clip;
+    below the bound nothing is written at all under either strategy."""
+    cpu = _grads([(300001,), (5,), (70000,), (6144,)], torch.float32, 1e-2, 1.0, seed=23)
+    dev = place_in_arena(cpu, DEV, 1, 1)
+    plan = TensorPlan(dev, dev)
+    plan.fused_step(1.0, max_norm, flags)
+    res = plan.result()
+    want = [g.clone() for g in cpu]
+    norm, coef = oracle.clip_grad_norm(want, max_norm)
+    assert math.isclose(res.norm, norm, rel_tol=REL)
+    assert res.clipped == (1 if coef is not None else 0)
+    for g, c, d in zip(cpu, want, dev):
+        if coef is None:
+            assert_bits_equal(d, g, "untouched")
+        else:
+            assert math.isclose(res.coef, coef, rel_tol=REL)
+            assert_bits_equal(d, g * torch.tensor(res.coef, dtype=torch.float32), "clipped in place")
+    plan.close()
+
+
+def test_max_norm_crosses_the_boundary_as_a_c_float():
+    """max_grad_norm = 0.1 is not an fp32 number: the reference narrows it at the binding
+    (``src/main.cpp:339-342``) and divides in double (``src/comp/ParamStorage.cpp:723-740``)."""
+    grads = _grads([(4097,), (33,)], torch.float32, 1.0, 1.0, seed=24)
+    res, tn, out = _run_fused(grads, torch.float32, 1.0, 0.1)
+    want = _check_against_oracle(grads, "f32", 1.0, 0.1, res, tn, out)
+    import numpy as np
+    assert want.coef == float(np.float32(0.1)) / (want.norm + 1e-6) and want.coef != 0.1 / (want.norm + 1e-6)
+    assert math.isclose(res.coef, float(np.float32(want.coef)), rel_tol=REL)

@@ -342,6 +342,63 @@ def test_amp_overflow_skips_the_step_and_halves_the_scale():
     assert oracle.patched_update_scale(want, True) is True and want.loss_scale == scaler.loss_scale()
 
 
+@pytest.mark.parametrize("fused", [False, True])
+def test_amp_keeps_one_device_table_across_steps(fused):
+    """The unscale table is created once: later steps re-point it (or find the gradients where they were)
+    instead of destroying and rebuilding it, and the model gradients are let go once their last reader is queued."""
+    model = _tiny_model()
+    opt = torch.optim.SGD(model.parameters(), lr=0.01)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, fused=fused)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    handles = set()
+    for step in range(5):
+        x = torch.randn(16, 32, device=DEV, dtype=torch.float16)
+        loss = rm(x).float().pow(2).mean()
+        with amp.scale_loss(loss, opt) as scaled:
+            scaled.backward()
+            if step == 2:       # make backward's next allocation land elsewhere: the table must follow, not be rebuilt
+                hold = [torch.empty_like(p.grad) for p in opt._amp_stash.all_fp16_params]
+        stash = opt._amp_stash
+        handles.add(stash.unscale_plan.plan._handle.value)
+        rm.clip_grad_norm(1.0)
+        opt.step()
+        assert all(s is None for s in stash.unscale_plan._srcs) and stash.pending_model_grads == []
+        opt.zero_grad()
+    assert len(handles) == 1
+    del hold
+
+
+@pytest.mark.parametrize("fused,fused_opt", [(False, False), (True, False), (True, True)])
+def test_amp_static_scale_overflow_reaches_the_parameters(fused, fused_opt):
+    """A static loss scale never skips a step (Apex): an overflow must not leave the previous step's master
+    gradients in place.  The inf lands in the master gradients, clipGradNorm's arithmetic turns it into NaN
+    (inf * (max / inf) = inf * 0), and the optimizer steps on that - in every mode."""
+    from rannc_amd.fused_optim import FusedSGD
+    model = _tiny_model()
+    opt = (FusedSGD if fused_opt else torch.optim.SGD)(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", loss_scale=128.0, fused=fused)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    x = torch.randn(16, 32, device=DEV, dtype=torch.float16)
+    for step in range(2):
+        loss = rm(x).float().pow(2).mean()
+        with amp.scale_loss(loss, opt) as scaled:
+            scaled.backward()
+            if step == 1:
+                opt._amp_stash.all_fp16_params[0].grad.view(-1)[3] = float("inf")
+        scaler = amp._amp_state.loss_scalers[0]
+        assert scaler.loss_scale() == 128.0
+        rm.clip_grad_norm(1e-3)
+        opt.step()
+        masters = opt._amp_stash.all_fp32_from_fp16_params
+        if step == 0:
+            assert all(bool(torch.isfinite(m).all()) for m in masters)
+        else:
+            assert opt._amp_stash.last_result.overflow == 1
+            assert not bool(torch.isfinite(masters[0]).all()), "the overflow was swallowed"
+            assert bool(torch.isnan(masters[0].view(-1)[3]))
+        opt.zero_grad()
+
+
 def test_patch_optimizer_zero_mode_bookkeeping():
     model = _tiny_model()
     opt = torch.optim.Adam(model.parameters(), lr=1e-3)

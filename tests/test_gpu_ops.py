@@ -256,6 +256,26 @@ def test_accumulate_and_unscale_accumulate(src_name, dst_name):
     plan.close()
 
 
+def test_unscale_accumulate_checks_the_incoming_gradients_only():
+    """Apex's unscale_with_stashed passes "check only arg 0, the incoming model grads" to its axpby kernel: an
+    inf already sitting in the stashed master gradient makes the result (and the norm) non-finite but does
+    not raise the flag."""
+    g = torch.Generator().manual_seed(19)
+    model = [(torch.randn(5000, generator=g) * 64.0).to(torch.float16), (torch.randn(300, generator=g) * 64.0).to(torch.float16)]
+    master = [torch.randn(5000, generator=g), torch.randn(300, generator=g)]
+    master[0][4321] = float("inf")
+    srcs, dsts = place_in_arena(model, DEV, 1, 3), place_in_arena(master, DEV, 2, 1)
+    plan = TensorPlan(srcs, dsts)
+    plan.unscale_accumulate(1.0 / 64.0)
+    res = plan.result()
+    want = [m.clone() for m in master]
+    assert oracle.unscale_accumulate(want, model, 1.0 / 64.0) == 0
+    assert res.overflow == 0 and math.isinf(res.norm)
+    for d, w in zip(dsts, want):
+        assert_bits_equal(d.cpu(), w, "accumulated onto a non-finite master gradient")
+    plan.close()
+
+
 @pytest.mark.parametrize("dst_name", ["f32", "bf16"])
 def test_chunk_boundaries_follow_the_destination_alignment(dst_name):
     """Chunk boundaries inside a tensor sit on 128-byte boundaries of its destination, so the
