@@ -164,6 +164,15 @@ int rg_step_decide(rg_plan* plan, float max_norm, int flags, void* stream);
  * clip.  Apex multi_tensor_scale semantics (LossScaler.unscale). */
 int rg_unscale_pack(rg_plan* plan, float inv_scale, void* stream);
 
+/* Clip after the fact: from the sums the last rg_unscale_pack / rg_unscale_accumulate on this plan left on
+ * the device, the clip decision for max_norm (as rg_fused_step takes it), and - only if it says "clip" - an
+ * in-place multiply of the destinations by the coefficient.  rg_unscale_pack + rg_step_apply_clip write the
+ * bits of rg_fused_step and move (s + d) bytes per element when the step does not clip, (s + 3d) when it
+ * does; the multiply's blocks cover whole chunks, so a launch that finds nothing to do costs microseconds.
+ * ParamStorage::clipGradNorm (src/comp/ParamStorage.cpp:721-745) on gradients whose norm is already known.
+ * RG_EINVAL unless the plan's last operation was one of the two named above. */
+int rg_step_apply_clip(rg_plan* plan, float max_norm, int flags, void* stream);
+
 /* Accumulating forms, for gradient accumulation over several backward passes:
  *   rg_accumulate:          dst = round_dst(float(dst) + float(src) * scale)
  *   rg_unscale_accumulate:  the same with scale = inv_scale, plus the inf/NaN flag of the sources

@@ -173,9 +173,11 @@ class RaNNCModule(_pyrannc.RaNNCModule):
                 if not any(p.grad is not None for p in stash.all_fp32_from_fp32_params):
                     finish_unscale(self.optimizer, max_f)
                     return
-            if stash is not None and stash.pending_finish:
-                from .amp import finish_unscale
                 finish_unscale(self.optimizer)
+            elif stash is not None:
+                from .amp import clip_from_unscale_sums
+                if clip_from_unscale_sums(self.optimizer, max_f):
+                    return
         super().clip_grad_norm(max_grad_norm)
 
     def _calc_grad_norm(self):

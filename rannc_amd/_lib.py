@@ -60,6 +60,7 @@ SIGNATURES = {
     "rg_step_finish": (_i, [_vp, _f, _i, _vp]),
     "rg_step_decide": (_i, [_vp, _f, _i, _vp]),
     "rg_unscale_pack": (_i, [_vp, _f, _vp]),
+    "rg_step_apply_clip": (_i, [_vp, _f, _i, _vp]),
     "rg_accumulate": (_i, [_vp, _f, _vp]),
     "rg_unscale_accumulate": (_i, [_vp, _f, _vp]),
     "rg_grad_norm": (_i, [_vp, _vp]),
@@ -217,6 +218,9 @@ class Plan:
 
     def unscale_pack(self, inv_scale: float, stream: int = 0) -> None:
         check(lib.rg_unscale_pack(self._handle, inv_scale, _vp(stream)))
+
+    def step_apply_clip(self, max_norm: float, flags: int = RG_STEP_DEFAULT, stream: int = 0) -> None:
+        check(lib.rg_step_apply_clip(self._handle, max_norm, flags, _vp(stream)))
 
     def accumulate(self, scale: float = 1.0, stream: int = 0) -> None:
         check(lib.rg_accumulate(self._handle, scale, _vp(stream)))

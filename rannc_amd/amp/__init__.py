@@ -53,6 +53,7 @@ class _AmpStash:
         self.lazy_init_called = False
         self.unscale_plan: Optional[TensorPlan] = None
         self.unscale_cache = None          # param_storage._PlanCache holding unscale_plan
+        self.optimizer_reads_model_grads = False    # a fused optimizer: its step kernel unscales and clips itself
         self.step_flags = _lib.RG_STEP_DEFAULT      # RG_STEP_IGNORE_OVERFLOW under a static loss scale
         self.copy_back_plan: Optional[TensorPlan] = None
         self.pending_finish = False        # fused mode: the write pass has not run yet
@@ -62,6 +63,12 @@ class _AmpStash:
         self.decided_max_norm: Optional[float] = None      # clip_grad_norm asked for while the write is pending
         self.fused = False
         self.last_result = None            # rg_step_result of the last unscale
+        # fused mode picks its strategy per step from what the last step did: when it clipped, read pass now and
+        # one deferred write pass that applies the coefficient ((2s + d) bytes per element); when it did not, one
+        # eager pass that writes while it sums ((s + d)), with an in-place multiply only if this step clips after all
+        self.expect_clip = True
+        self.clip_decided = False          # a clip decision was taken on the device since the last unscale
+        self.sums_cover_all = False        # the eager pass's sums are the norm of every gradient clip_grad_norm covers
         # packed fp32 bucket the master gradients are views of (the reference's
         # consolidated_master_grads_, src/comp/ParamStorage.cpp:68-70, 92-97): stable
         # addresses, so the device table is built once
@@ -107,16 +114,22 @@ class LossScaler:
             stash.unscale_cache = _PlanCache()
         stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads)
         inv = 1.0 / self._loss_scale
+        if stash.clip_decided:
+            # what the last step decided (still in the table's result block) picks this step's strategy
+            stash.expect_clip = bool(stash.unscale_plan.result().clipped)
+            stash.clip_decided = False
+        stash.sums_cover_all = False
         with torch.no_grad():
             if accumulate:
                 stash.unscale_plan.unscale_accumulate(inv)
-            elif stash.fused:
+            elif stash.fused and (stash.expect_clip or stash.optimizer_reads_model_grads):
                 stash.unscale_plan.step_begin(inv)
                 stash.pending_finish = True
                 stash.pending_inv_scale = inv
                 stash.decided_max_norm = None
             else:
                 stash.unscale_plan.unscale_pack(inv)
+                stash.sums_cover_all = stash.fused
         stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
         if stash.last_result.overflow:
             self._has_overflow = True
@@ -145,22 +158,26 @@ class LossScaler:
 
 def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_level: str = "O2",
                loss_scale="dynamic", max_loss_scale: float = 2.0 ** 24, min_loss_scale: Optional[float] = None,
-               half_dtype: torch.dtype = torch.float16, fused: bool = False
+               half_dtype: torch.dtype = torch.float16, fused: bool = True
                ) -> Tuple[torch.nn.Module, torch.optim.Optimizer]:
     """O2-style set-up: the model's floating-point parameters (batch-norm layers excepted)
     become ``half_dtype``; the optimizer is re-pointed at fp32 masters created as
     ``param.detach().clone().float()``; ``optimizer.step`` is wrapped to skip once after an
     overflow and to copy masters back into the model afterwards.
 
-    ``fused=True`` defers the write of the unscaled master gradients from the ``scale_loss``
-    exit to the next ``clip_grad_norm`` / ``optimizer.step``, so that unscale, norm, clip and
-    pack move ``(2s + d)`` bytes per element; until then master ``.grad`` holds stale data.
+    ``fused=True`` (the default) defers the write of the unscaled master gradients from the ``scale_loss``
+    exit to the next ``clip_grad_norm`` / ``optimizer.step``, so that unscale, norm, clip and pack move
+    ``(2s + d)`` bytes per element (``(s + d)`` when the previous step did not clip) instead of the
+    ``(s + d) + 3d`` of an eager unscale followed by a clip of the fp32 gradients.  Everything that hands
+    master gradients out - ``amp.master_params``, ``RaNNCModule.get_param_grad`` / ``_calc_grad_norm`` /
+    ``clip_grad_norm``, ``optimizer.step`` - completes the write first; only code that reaches into
+    ``optimizer._amp_stash`` directly sees stale values until then (call ``amp.finish_unscale(optimizer)``).
+    ``fused=False`` writes them at the ``scale_loss`` exit, as Apex does.
     When the optimizer is one of ``rannc_amd.fused_optim`` (and every stepped parameter is half
     precision) the write never happens: ``clip_grad_norm`` only takes the clip decision on the
     device and ``optimizer.step`` reads the scaled model gradients, applies ``1/scale`` and the
     clip coefficient, updates the masters and writes the model copies in one kernel.  Anything
-    that looks at master gradients first (``calc_grad_norm``, ``get_param_grad``,
-    ``finish_unscale``) writes them, and the step then takes them from memory."""
+    that looks at master gradients first writes them, and the step then takes them from memory."""
     if opt_level != "O2":
         raise ValueError("only opt_level='O2' (fp32 masters for half parameters) is provided")
     bn = torch.nn.modules.batchnorm._BatchNorm
@@ -175,6 +192,7 @@ def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_lev
                 mod._buffers[name] = b.to(half_dtype)
     stash = _AmpStash()
     stash.fused = fused
+    stash.optimizer_reads_model_grads = bool(getattr(optimizer, "reads_grad_sources", False))
     optimizer._amp_stash = stash
     scaler = LossScaler(loss_scale, min_loss_scale=min_loss_scale, max_loss_scale=max_loss_scale)
     # A static scale never skips a step (Apex): an overflow must then reach the master gradients and the
@@ -218,7 +236,12 @@ def _lazy_init_maybe_master_weights(optimizer: torch.optim.Optimizer) -> None:
 
 
 def master_params(optimizer: torch.optim.Optimizer) -> Iterator[torch.Tensor]:
-    """``apex.amp.master_params``: every parameter the optimizer steps on."""
+    """``apex.amp.master_params``: every parameter the optimizer steps on.  Callers use it to get at the
+    master gradients (``clip_grad_norm_(amp.master_params(optimizer), ...)``), so a deferred write of
+    those gradients is completed first."""
+    stash = getattr(optimizer, "_amp_stash", None)
+    if stash is not None and stash.pending_finish:
+        finish_unscale(optimizer)
     for group in optimizer.param_groups:
         for p in group["params"]:
             yield p
@@ -233,6 +256,7 @@ def finish_unscale(optimizer: torch.optim.Optimizer, max_norm: Optional[float] =
             max_norm = stash.decided_max_norm or 0.0
         with torch.no_grad():
             stash.unscale_plan.step_finish(float(max_norm), stash.step_flags)
+        stash.clip_decided = True
         stash.pending_finish = False
         stash.decided_max_norm = None
         stash.unscale_plan.drop_sources()
@@ -255,7 +279,22 @@ def decide_clip(optimizer: torch.optim.Optimizer, max_norm: float) -> None:
     stash = optimizer._amp_stash
     with torch.no_grad():
         stash.unscale_plan.step_decide(float(max_norm), stash.step_flags)
+    stash.clip_decided = True
     stash.decided_max_norm = float(max_norm)
+
+
+def clip_from_unscale_sums(optimizer: torch.optim.Optimizer, max_norm: float) -> bool:
+    """Fused mode after an eager unscale: the norm of the master gradients is already on the device, so clipping
+    is the decision plus - only if it says "clip" - one in-place multiply.  Returns False when those sums do not
+    cover every gradient ``clip_grad_norm`` is about (fp32 parameters with gradients, accumulation)."""
+    stash = optimizer._amp_stash
+    if not stash.sums_cover_all or any(p.grad is not None for p in stash.all_fp32_from_fp32_params):
+        return False
+    with torch.no_grad():
+        stash.unscale_plan.step_apply_clip(float(max_norm), stash.step_flags)
+    stash.sums_cover_all = False
+    stash.clip_decided = True
+    return True
 
 
 def _master_to_model(optimizer: torch.optim.Optimizer) -> None:
@@ -470,6 +509,13 @@ def patch_amp_scaler():
 
 
 def unset_master_grads(optimizer):
-    """``pyrannc/amp/__init__.py:68-70``."""
-    for p in master_params(optimizer):
-        p.grad = None
+    """``pyrannc/amp/__init__.py:68-70``: drop every master gradient (a write that was still deferred with them)."""
+    stash = getattr(optimizer, "_amp_stash", None)
+    if stash is not None and stash.pending_finish:
+        stash.pending_finish = False
+        stash.decided_max_norm = None
+        stash.unscale_plan.drop_sources()
+        stash.pending_model_grads = []
+    for group in optimizer.param_groups:
+        for p in group["params"]:
+            p.grad = None

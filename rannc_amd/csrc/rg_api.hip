@@ -42,6 +42,7 @@ struct rg_plan {
   int xcd_write_offgrid = 256;       //   ... when some source does not (see fill_chunk_records)
   int64_t reduce_tile_factor = 0;    // tile of a reducing + writing pass, in write tiles (0 = per operation)
   float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
+  bool sums_describe_dst = false;   // the per-tensor sums on the device are those of the destinations as last written
   std::vector<TensorDesc> host_tensors;
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
   bool dst_heads = false;            // some destination starts off a 128-byte boundary
@@ -362,6 +363,7 @@ RG_API int rg_plan_update_pointers(rg_plan* p, const void* const* src, void* con
     if (src) p->host_tensors[(size_t)i].src = src[i];
     if (dst) p->host_tensors[(size_t)i].dst = dst[i];
   }
+  if (dst) p->sums_describe_dst = false;
   if (p->n_chunks == 0) return RG_OK;
   DeviceGuard guard(p->device);
   const int k = p->next_stage;
@@ -491,6 +493,7 @@ static int check_plan(const rg_plan* p, int need, const char* op) {
 RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags, void* stream) {
   const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_fused_step");
   if (rc != RG_OK) return rc;
+  p->sums_describe_dst = false;
   if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
     set_error("rg_fused_step: inv_scale must be a non-zero number");
     return RG_EINVAL;
@@ -542,6 +545,7 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
 RG_API int rg_step_begin(rg_plan* p, float inv_scale, void* stream) {
   const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_step_begin");
   if (rc != RG_OK) return rc;
+  p->sums_describe_dst = false;
   if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
     set_error("rg_step_begin: inv_scale must be a non-zero number");
     return RG_EINVAL;
@@ -598,7 +602,28 @@ RG_API int rg_unscale_pack(rg_plan* p, float inv_scale, void* stream) {
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, inv_scale);
-  return tiled_reduce_write(p, a, kModeReduce | kModeWrite, s);
+  const int rc2 = tiled_reduce_write(p, a, kModeReduce | kModeWrite, s);
+  p->sums_describe_dst = rc2 == RG_OK;
+  return rc2;
+}
+
+RG_API int rg_step_apply_clip(rg_plan* p, float max_norm, int flags, void* stream) {
+  const int rc = check_plan(p, kNeedDst, "rg_step_apply_clip");
+  if (rc != RG_OK) return rc;
+  if (!p->sums_describe_dst) {
+    set_error("rg_step_apply_clip: the last operation on this plan was not rg_unscale_pack / rg_unscale_accumulate");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  RG_HIP(launch_finalize_total(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
+  PassArgs b = pass_args(p, 1.0f);
+  b.result = p->d_result;
+  b.only_if_clipped = 1;
+  b.src_is_dst = 1;
+  RG_HIP(launch_pass(kModeWrite, b, p->streaming, s));   // one block per chunk: cheap to find idle
+  p->sums_describe_dst = false;                          // the destinations are about to change
+  return RG_OK;
 }
 
 static int check_not_in_place(const rg_plan* p, const char* op) {
@@ -616,6 +641,7 @@ RG_API int rg_accumulate(rg_plan* p, float scale, void* stream) {
   int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_accumulate");
   if (rc == RG_OK) rc = check_not_in_place(p, "rg_accumulate");
   if (rc != RG_OK) return rc;
+  p->sums_describe_dst = false;
   DeviceGuard guard(p->device);
   PassArgs a = pass_args(p, scale);
   split_for_write(p, a);
@@ -634,12 +660,15 @@ RG_API int rg_unscale_accumulate(rg_plan* p, float inv_scale, void* stream) {
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, inv_scale);
-  return tiled_reduce_write(p, a, kModeReduce | kModeWrite | kModeAccumulate, s);
+  const int rc2 = tiled_reduce_write(p, a, kModeReduce | kModeWrite | kModeAccumulate, s);
+  p->sums_describe_dst = rc2 == RG_OK;
+  return rc2;
 }
 
 RG_API int rg_grad_norm(rg_plan* p, void* stream) {
   const int rc = check_plan(p, kNeedSrc, "rg_grad_norm");
   if (rc != RG_OK) return rc;
+  p->sums_describe_dst = false;
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, 1.0f);
@@ -653,6 +682,7 @@ RG_API int rg_grad_norm(rg_plan* p, void* stream) {
 RG_API int rg_scale_cast(rg_plan* p, float scale, void* stream) {
   const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_scale_cast");
   if (rc != RG_OK) return rc;
+  p->sums_describe_dst = false;
   DeviceGuard guard(p->device);
   PassArgs a = pass_args(p, scale);
   split_for_write(p, a);
@@ -828,6 +858,7 @@ RG_API int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t nume
 RG_API int rg_zero(rg_plan* p, void* stream) {
   const int rc = check_plan(p, kNeedDst, "rg_zero");
   if (rc != RG_OK) return rc;
+  p->sums_describe_dst = false;
   DeviceGuard guard(p->device);
   PassArgs a = pass_args(p, 1.0f);
   a.zero_fill = 1;

@@ -140,6 +140,9 @@ class TensorPlan:
     def unscale_pack(self, inv_scale: float) -> None:
         self.plan.unscale_pack(inv_scale, self._stream())
 
+    def step_apply_clip(self, max_norm: float, flags: int = _lib.RG_STEP_DEFAULT) -> None:
+        self.plan.step_apply_clip(max_norm, flags, self._stream())
+
     def accumulate(self, scale: float = 1.0) -> None:
         self.plan.accumulate(scale, self._stream())
 

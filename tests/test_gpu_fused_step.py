@@ -297,3 +297,23 @@ def test_max_norm_crosses_the_boundary_as_a_c_float():
     import numpy as np
     assert want.coef == float(np.float32(0.1)) / (want.norm + 1e-6) and want.coef != 0.1 / (want.norm + 1e-6)
     assert math.isclose(res.coef, float(np.float32(want.coef)), rel_tol=REL)
+
+
+@pytest.mark.parametrize("max_norm", [0.5, 1e9])
+def test_unscale_pack_then_apply_clip_writes_the_bits_of_the_fused_step(max_norm):
+    grads = _grads([(300001,), (5,), (70000,), (6144,)], torch.bfloat16, 1e-2, 65536.0, seed=25)
+    srcs = place_in_arena(grads, DEV, 1, 1)
+    total = sum(g.numel() for g in grads)
+    bucket = torch.full((total + 3,), 7.0, dtype=torch.float32, device=DEV)[3:]
+    offs, _ = oracle.bucket_layout([g.numel() for g in grads], ["f32"] * len(grads))
+    dsts = [bucket.narrow(0, o, g.numel()) for o, g in zip(offs, grads)]
+    plan = TensorPlan(srcs, dsts)
+    with pytest.raises(ValueError, match="rg_unscale_pack"):
+        plan.step_apply_clip(max_norm)                      # nothing has left sums of the destinations yet
+    plan.unscale_pack(1 / 65536.0)
+    plan.step_apply_clip(max_norm)
+    res, tn = plan.result(), plan.tensor_norms()
+    _check_against_oracle(grads, "f32", 1 / 65536.0, max_norm, res, tn, bucket.cpu())
+    with pytest.raises(ValueError, match="rg_unscale_pack"):
+        plan.step_apply_clip(max_norm)                      # the sums no longer describe the destinations
+    plan.close()

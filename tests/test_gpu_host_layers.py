@@ -563,3 +563,55 @@ def test_scale_loss_restores_stashed_gradients_when_the_body_raises():
         with amp.scale_loss(rm(x).float().sum(), opt) as scaled:
             raise RuntimeError("boom")
     assert torch.equal(model[1].weight.grad, kept)
+
+
+def test_amp_fused_mode_picks_its_strategy_from_the_last_step():
+    """Default (fused) amp: a step after one that clipped defers the write and applies the coefficient in it; a
+    step after one that did not clip writes eagerly while summing and multiplies in place only if it clips after
+    all.  Either way the master gradients are the oracle's: unscale, then clip by the norm."""
+    model = _tiny_model()
+    opt = torch.optim.SGD(model.parameters(), lr=0.0)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    stash = opt._amp_stash
+    assert stash.fused
+    seen = []
+    #            bound     deferred write expected at this step
+    for bound, deferred in ((1e9, True), (1e9, False), (1e-3, False), (1e-3, True), (1e9, True), (1e-3, False)):
+        x = torch.randn(16, 32, device=DEV, dtype=torch.float16)
+        loss = rm(x).float().pow(2).mean()
+        with amp.scale_loss(loss, opt) as scaled:
+            scaled.backward()
+            grads = [p.grad.detach().cpu().clone() for p in stash.all_fp16_params]
+        assert stash.pending_finish == deferred
+        seen.append(stash.pending_finish)
+        rm.clip_grad_norm(bound)
+        want, flag = oracle.unscale_and_check(grads, 1.0 / 256.0)
+        norm, coef = oracle.clip_grad_norm(want, bound)
+        assert flag == 0 and (coef is not None) == (bound == 1e-3)
+        res = stash.unscale_plan.result()
+        assert res.clipped == (1 if coef is not None else 0) and math.isclose(res.norm, norm, rel_tol=1e-6)
+        unscaled, _ = oracle.unscale_and_check(grads, 1.0 / 256.0)
+        for m, u in zip(stash.all_fp32_from_fp16_params, unscaled):
+            assert_bits_equal(m.grad.cpu(), u * torch.tensor(res.coef) if res.clipped else u, "master gradient")
+        opt.step()
+        opt.zero_grad()
+    assert seen == [True, False, False, True, True, False]
+
+
+def test_amp_master_params_completes_a_deferred_write():
+    model = _tiny_model()
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    x = torch.randn(16, 32, device=DEV, dtype=torch.float16)
+    loss = rm(x).float().pow(2).mean()
+    with amp.scale_loss(loss, opt) as scaled:
+        scaled.backward()
+        grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
+    assert opt._amp_stash.pending_finish
+    masters = list(amp.master_params(opt))          # the Apex recipe: clip_grad_norm_(amp.master_params(optimizer), ...)
+    assert not opt._amp_stash.pending_finish
+    want, _ = oracle.unscale_and_check(grads, 1.0 / 256.0)
+    for m, w in zip(masters, want):
+        assert_bits_equal(m.grad.cpu(), w, "master gradient handed out by master_params")

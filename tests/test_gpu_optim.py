@@ -175,12 +175,13 @@ def test_gate_applies_the_clip_coefficient_and_skips_on_overflow():
         close(a, b, 1e-9, "grad_scale")
 
 
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("half", [torch.float16, torch.bfloat16])
-def test_amp_with_fused_adam_writes_model_copies_from_the_step(half):
+def test_amp_with_fused_adam_writes_model_copies_from_the_step(half, fused):
     torch.manual_seed(3)
     model = torch.nn.Sequential(torch.nn.Linear(32, 48), torch.nn.Tanh(), torch.nn.Linear(48, 8)).to(DEV)
     opt = FusedAdam(model.parameters(), lr=1e-2)
-    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, half_dtype=half)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, half_dtype=half, fused=fused)
     rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
     masters_before = None
     for it in range(3):
@@ -188,11 +189,16 @@ def test_amp_with_fused_adam_writes_model_copies_from_the_step(half):
         loss = rm(x).float().pow(2).mean()
         with amp.scale_loss(loss, opt) as scaled:
             scaled.backward()
+            model_grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
         stash = opt._amp_stash
         assert getattr(stash, "optimizer_copies_back", False) and stash.copy_back_plan is None
         masters = stash.all_fp32_from_fp16_params
         m_cpu = [m.detach().cpu().clone() for m in masters]
-        g_cpu = [m.grad.detach().cpu().clone() for m in masters]
+        if fused:       # the master gradients are never written: the step kernel unscales the model gradients itself
+            assert stash.pending_finish
+            g_cpu, _ = oracle.unscale_and_check(model_grads, 1.0 / 256.0)
+        else:
+            g_cpu = [m.grad.detach().cpu().clone() for m in masters]
         ms = [opt.state[m]["exp_avg"].cpu().clone() if m in opt.state and len(opt.state[m]) else torch.zeros_like(c) for m, c in zip(masters, m_cpu)]
         vs = [opt.state[m]["exp_avg_sq"].cpu().clone() if m in opt.state and len(opt.state[m]) else torch.zeros_like(c) for m, c in zip(masters, m_cpu)]
         opt.step()
@@ -200,6 +206,7 @@ def test_amp_with_fused_adam_writes_model_copies_from_the_step(half):
         for m, want, p in zip(masters, m_cpu, stash.all_fp16_params):
             close(m, want, 1e-2 * RTOL, f"master it {it}")
             assert_bits_equal(p.detach().cpu(), oracle_optim.model_copy(m.detach().cpu(), half), "model copy written by the step")
+        opt.zero_grad()
         rm.zero_grad()
     assert stash.copy_back_plan is None                   # the separate copy-back pass never ran
 
