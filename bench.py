@@ -31,7 +31,7 @@ FUSED_OPS = ("fused_step", "fused_step_noclip", "fused_step_noclip_2pass", "over
              "copy_back", "unflatten_back", "grad_norm", "zero")
 C5_OPS = ("c5_unflatten", "c5_master_cast", "c5_copy_back", "c5_repack")
 OPTIM_OPS = ("adam", "sgd", "adam_from_model_grads")
-ALL_OPS = ("all",) + FUSED_OPS + C5_OPS + OPTIM_OPS
+ALL_OPS = ("all",) + FUSED_OPS + C5_OPS + OPTIM_OPS + ("api_step",)
 
 
 def parse_args():
@@ -513,6 +513,115 @@ def cpu_baseline_optimizer(op: str, shapes, seed: int, budget_s: float, bytes_pe
                       f"torch.optim's per-tensor op sequence + master->bf16 copy"}
 
 
+# ----------------------------------------------------------------------------- the drop-in API path
+
+def bench_api_step(args, key: str) -> dict:
+    full = _api_step_leg(args, key, 1.0)
+    # the same tensor list with every tensor cut to one row: the kernels have next to nothing to do, so the wall
+    # time of a step is the host's own cost of driving the API (including its one wait for the flag per step)
+    tiny = _api_step_leg(args, key, 0.0)
+    full["host_only"] = {"what": "same calls on the same tensor list with every tensor cut to one row of dim 0",
+                         "elements": tiny["config"]["elements"], "us_per_step": tiny["value"],
+                         "device_us_per_step": tiny["device_us_per_step"], "us_per_call": tiny["host_us_per_call"]}
+    full["host_us_per_step"] = tiny["value"]
+    full["host_fraction_of_device_time"] = round(tiny["value"] / full["device_us_per_step"], 3)
+    return full
+
+
+def _api_step_leg(args, key: str, scale_numel: float) -> dict:
+    """Host time of the path a training script drives, on a parameter list shaped like ``key``: the exit of
+    ``amp.scale_loss`` (unscale + flag), ``RaNNCModule.clip_grad_norm``, ``FusedAdam.step`` and ``zero_grad``.
+    Backward is replaced by handing every half parameter a ready gradient tensor.  Reports wall microseconds per
+    call (host + device, the host waits for the flag at the scale_loss exit as the reference does) next to the
+    device time of the same step, and the host time alone of every call (measured with the device idle-waiting
+    excluded: time until the call returns)."""
+    import torch
+    import rannc_amd
+    from rannc_amd import amp
+    from rannc_amd.fused_optim import FusedAdam
+    from rannc_amd.workloads import step_config
+
+    cfg = step_config(key)
+    dev = torch.device("cuda", 0)
+    half = torch.bfloat16
+
+    class Holder(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            shapes = [sh if scale_numel >= 1.0 else (max(1, int(sh[0] * scale_numel)),) + tuple(sh[1:]) for _, sh in cfg.params]
+            self.ps = torch.nn.ParameterList([torch.nn.Parameter(torch.randn(sh, device=dev) * 0.02) for sh in shapes])
+
+        def forward(self, x):
+            return x
+
+    model = Holder()
+    opt = FusedAdam(model.parameters(), lr=1e-4)
+    model, opt = amp.initialize(model, opt, opt_level="O2", half_dtype=half, loss_scale=65536.0)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    rm._deploy()
+    params = list(model.parameters())
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    grads = [(torch.randn(p.shape, device=dev, generator=gen) * 1e-2 * 65536.0).to(half) for p in params]
+    n = sum(p.numel() for p in params)
+    loss = torch.zeros((), device=dev)
+    names = ("assign_grads", "scale_loss_exit", "clip_grad_norm", "optimizer_step", "zero_grad")
+    host = {k: 0.0 for k in names}
+
+    def one_step(record: bool):
+        t = [time.perf_counter()]
+        ctx = amp.scale_loss(loss, opt)
+        ctx.__enter__()
+        for p, g in zip(params, grads):
+            p.grad = g
+        t.append(time.perf_counter())
+        ctx.__exit__(None, None, None)
+        t.append(time.perf_counter())
+        rm.clip_grad_norm(1.0)
+        t.append(time.perf_counter())
+        opt.step()
+        t.append(time.perf_counter())
+        opt.zero_grad()
+        rm.zero_grad()
+        t.append(time.perf_counter())
+        if record:
+            for k, a, b in zip(names, t[:-1], t[1:]):
+                host[k] += b - a
+
+    for _ in range(max(args.warmup, 10)):
+        one_step(False)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        one_step(True)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / args.steps
+    dev_s = e0.elapsed_time(e1) * 1e-3 / args.steps
+    # device time of the kernels alone: the same launches back to back, nothing read on the host in between
+    stash = opt._amp_stash
+    bytes_per_elem = 2 + (2 + 12) + (12 + 2)     # read pass; Adam reading the scaled gradient; p, m, v and the model copy out
+    out = {
+        "metric": "host microseconds per training step through the RaNNCModule / amp / FusedAdam API",
+        "value": round(wall * 1e6, 1), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 model / f32 masters", "data": "synthetic",
+        "config": {"workload": key, "op": "api_step", "tensors": len(params), "elements": n, "seed": args.seed,
+                   "deferred_write": bool(stash.fused), "optimizer": "FusedAdam"},
+        "device_us_per_step": round(dev_s * 1e6, 1),
+        "host_us_per_call": {k: round(v / args.steps * 1e6, 1) for k, v in host.items()},
+        "host_us_per_step_without_assign": round(sum(v for k, v in host.items() if k != "assign_grads") / args.steps * 1e6, 1),
+        "algorithmic_bytes_per_step": bytes_per_elem * n,
+        "GB/s": round(bytes_per_elem * n / wall / 1e9, 1),
+        "note": "scale_loss_exit includes the wait for the overflow flag (one host read per step, as the reference's .item())",
+    }
+    rm.undeploy()
+    del model, opt, rm, params, grads
+    torch.cuda.empty_cache()
+    return out
+
+
 # ----------------------------------------------------------------------------- main
 
 def headline_line(args, e: dict, w_desc: dict, dtype: str) -> dict:
@@ -579,6 +688,10 @@ def main() -> int:
     everything = args.op in (None, "all") and args.workload is None
     if args.op in OPTIM_OPS:
         print(json.dumps(bench_optimizer(args, args.workload or "c2_bert_large", torch, dev)), flush=True)
+        return 0
+
+    if args.op == "api_step":
+        print(json.dumps(bench_api_step(args, args.workload or "c4_resnet152x2")), flush=True)
         return 0
 
     key = args.workload or HEADLINE

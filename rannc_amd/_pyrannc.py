@@ -113,6 +113,13 @@ def dist_param_registered(pid: int) -> bool:
     return _dist_param_locator.registered(pid)
 
 
+def gather_tensor_zero(ten: torch.Tensor, pid: int) -> torch.Tensor:
+    """``src/main.cpp`` ``gather_tensor_zero`` -> ``ParamStorage::gatherTensorZero``
+    (``src/comp/ParamStorage.cpp:670-685``): the per-rank pieces of a tensor laid out like the ZeRO
+    segments of parameter ``pid``, gathered and viewed in the parameter's shape."""
+    return _param_storage.gather_tensor_zero(ten, pid)
+
+
 def get_param_ranks(pid: int):
     _param_storage.get_param_tensor(pid)
     return {0}

@@ -102,17 +102,22 @@ class LossScaler:
         self._has_overflow = False
 
     def unscale(self, stash: _AmpStash, model_grads: List[torch.Tensor], master_grads: List[torch.Tensor],
-                accumulate: bool = False) -> None:
+                accumulate: bool = False, all_params: bool = False) -> None:
         """``master_grad = float(model_grad) * (1 / scale)`` for every pair in one launch, with the
         inf/NaN flag and - for free - the gradient norm.  In fused mode only the read pass runs
         here; the values are written by ``finish_unscale``.  ``accumulate`` adds to the master
-        gradients instead of overwriting them (always eager)."""
+        gradients instead of overwriting them (always eager).  ``all_params``: the lists are every half
+        parameter's gradient and every master's bucket view, in stash order - the shape of the table is then known
+        to be last time's and only the gradients' addresses are compared."""
         # One device table for the whole run: when backward hands back gradients at new addresses (same
         # sizes and dtypes) the table is re-pointed in place, stream ordered - nothing is freed or allocated.
         if stash.unscale_cache is None:
             from ..param_storage import _PlanCache
             stash.unscale_cache = _PlanCache()
-        stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads)
+        if all_params:
+            stash.unscale_plan = stash.unscale_cache.get_same_shapes("all", model_grads, master_grads)
+        else:
+            stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads)
         inv = 1.0 / self._loss_scale
         if stash.clip_decided:
             # what the last step decided (still in the table's result block) picks this step's strategy
@@ -382,31 +387,44 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
         stash.master_grad_bucket = torch.empty(lens[_lib.RG_F32], dtype=torch.float32, device=masters[0].device)
         stash.master_grad_views = [stash.master_grad_bucket.narrow(0, o, m.numel()).view(m.shape)
                                    for o, m in zip(offs, masters)]
-    fresh, live = [], []
-    for i, (p, m) in enumerate(zip(stash.all_fp16_params, stash.all_fp32_from_fp16_params)):
-        if p.grad is None:
-            continue
-        (fresh if m.grad is None else live).append(i)
-    accumulate = bool(live)
-    if accumulate:
-        finish_unscale(optimizer)                 # a deferred write must land before it is added to
-        from ..multi_tensor import fill_zero_
-        for i in fresh:                           # mixed case: start the missing ones from zero
-            m = stash.all_fp32_from_fp16_params[i]
-            m.grad = stash.master_grad_views[i]
-            fill_zero_(m.grad.view(-1)) if m.grad.is_contiguous() else m.grad.zero_()
-    masters = []
-    for i in sorted(fresh + live):
-        p, m = stash.all_fp16_params[i], stash.all_fp32_from_fp16_params[i]
-        if m.grad is None:
-            m.grad = stash.master_grad_views[i]
-        model_grads.append(p.grad)
-        master_grads.append(m.grad)
-        masters.append(m)
-    stash.pending_masters, stash.pending_model_grads = masters, list(model_grads)
+    half_params, masters_all = stash.all_fp16_params, stash.all_fp32_from_fp16_params
+    model_grads_all = [p.grad for p in half_params]
+    n_with_grad = sum(1 for g in model_grads_all if g is not None)
+    n_live = sum(1 for m in masters_all if m.grad is not None)
     scaler.clear_overflow_state()
-    if model_grads:
-        scaler.unscale(stash, model_grads, master_grads, accumulate=accumulate)
+    if n_with_grad == len(half_params) and n_live == 0 and half_params:
+        # The steady state of a training loop: every half parameter has a fresh gradient and no master gradient
+        # is alive (zero_grad dropped them).  Nothing is classified or sorted; the table keeps its shape.
+        views = stash.master_grad_views
+        for m, v in zip(masters_all, views):
+            m.grad = v
+        stash.pending_masters, stash.pending_model_grads = masters_all, model_grads_all
+        scaler.unscale(stash, model_grads_all, views, accumulate=False, all_params=True)
+    else:
+        fresh, live = [], []
+        for i, (g, m) in enumerate(zip(model_grads_all, masters_all)):
+            if g is None:
+                continue
+            (fresh if m.grad is None else live).append(i)
+        accumulate = bool(live)
+        if accumulate:
+            finish_unscale(optimizer)                 # a deferred write must land before it is added to
+            from ..multi_tensor import fill_zero_
+            for i in fresh:                           # mixed case: start the missing ones from zero
+                m = masters_all[i]
+                m.grad = stash.master_grad_views[i]
+                fill_zero_(m.grad.view(-1)) if m.grad.is_contiguous() else m.grad.zero_()
+        masters = []
+        for i in sorted(fresh + live):
+            m = masters_all[i]
+            if m.grad is None:
+                m.grad = stash.master_grad_views[i]
+            model_grads.append(model_grads_all[i])
+            master_grads.append(m.grad)
+            masters.append(m)
+        stash.pending_masters, stash.pending_model_grads = masters, list(model_grads)
+        if model_grads:
+            scaler.unscale(stash, model_grads, master_grads, accumulate=accumulate)
     # fp32 parameters keep their own .grad; it carries the loss scale too
     from ..param_storage import _PlanCache
     if stash.fp32_unscale_plans is None:
@@ -444,67 +462,69 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
 # --------------------------------------------------------------------------- reference API
 
 def zip_params(optimizer):
+    """(fp32 master, half model parameter) pairs in stash order (``pyrannc/amp/__init__.py:9-11``); creates the
+    masters first if no ``scale_loss`` has run yet."""
     _lazy_init_maybe_master_weights(optimizer)
     stash = optimizer._amp_stash
     return zip(stash.all_fp32_from_fp16_params, stash.all_fp16_params)
 
 
 def register_amp_params(optimizer):
-    """``pyrannc/amp/__init__.py:13-18``."""
-    for master_p, model_p in zip_params(optimizer):
-        if model_p in getattr(optimizer, "param_zero_segment_to_id", {}):
-            _pyrannc.register_amp_master_param(optimizer.param_zero_segment_to_id[model_p], master_p)
-        else:
-            _pyrannc.register_amp_master_param(id(model_p), master_p)
+    """Tell the registry which fp32 master belongs to which model parameter (``pyrannc/amp/__init__.py:13-18``).
+    Under ZeRO the optimizer holds local segments; they are registered under the id of the parameter they are
+    a segment of."""
+    segment_owner = getattr(optimizer, "param_zero_segment_to_id", {})
+    for master, model_param in zip_params(optimizer):
+        owner = segment_owner[model_param] if model_param in segment_owner else id(model_param)
+        _pyrannc.register_amp_master_param(owner, master)
 
 
 def named_master_params(model, optimizer, zero=False):
-    """``pyrannc/amp/__init__.py:21-41``."""
-    if hasattr(optimizer._amp_stash, "all_fp32_from_fp16_params"):
-        amp_param_map = {model_p: master_p for master_p, model_p in zip_params(optimizer)}
-        if zero:
-            pid_to_name = {pid: n for n, pid in model.name_to_pid.items()}
-            pid_to_segment = {pid: segment for segment, pid in optimizer.param_zero_segment_to_id.items()}
-            for pid, segment in pid_to_segment.items():
-                if segment.dtype == torch.float:
-                    amp_param_map[segment] = segment
-            for model_p, master_p in amp_param_map.items():
-                yield pid_to_name[optimizer.param_zero_segment_to_id[model_p]], master_p
-        else:
-            for p in model.parameters():
-                if p.dtype == torch.float:
-                    amp_param_map[p] = p
-            for n, p in model.named_parameters():
-                yield n, amp_param_map[p]
+    """``(name, tensor the optimizer steps on)`` for every parameter (``pyrannc/amp/__init__.py:21-41``): the
+    fp32 master of a half parameter, the parameter itself when it already is fp32.  With ``zero`` the tensors
+    are local segments and the names come from the module's ``name_to_pid``; otherwise the order is that of
+    ``model.named_parameters()``."""
+    if not hasattr(optimizer._amp_stash, "all_fp32_from_fp16_params"):
+        return
+    stepped_for = {model_param: master for master, model_param in zip_params(optimizer)}
+    if zero:
+        name_of = {pid: name for name, pid in model.name_to_pid.items()}
+        for segment in optimizer.param_zero_segment_to_id:
+            if segment.dtype == torch.float:
+                stepped_for[segment] = segment
+        for model_param, master in stepped_for.items():
+            yield name_of[optimizer.param_zero_segment_to_id[model_param]], master
+    else:
+        for p in model.parameters():
+            if p.dtype == torch.float:
+                stepped_for[p] = p
+        for name, p in model.named_parameters():
+            yield name, stepped_for[p]
 
 
 def patch_amp_scaler():
-    """``pyrannc/amp/__init__.py:44-65``: after the scaler's own ``update_scale`` share the
-    overflow flag (sum over ranks) and, on overflow anywhere, adopt the smallest loss scale."""
+    """Make the loss scaler's ``update_scale`` a collective decision (``pyrannc/amp/__init__.py:44-65``): the
+    scaler's own update runs first; the overflow flag is summed over all ranks as an int32 on the device; if
+    any rank overflowed, every rank adopts the smallest ``int(loss_scale)``, restarts its count of clean steps
+    and reports that the step must be skipped."""
     scaler = _amp_state.loss_scalers[0]
     if getattr(scaler, "_rannc_patched", False):
         return
+    own_update = scaler.update_scale
 
-    def decorate(func):
-        def wrapper():
-            had_overflow = func()
-
-            # Share if overflow happens on any of ranks
-            flag_overflow = torch.IntTensor([0]).cuda()
-            if had_overflow:
-                flag_overflow = torch.IntTensor([1]).cuda()
-            _allreduce_sum(flag_overflow)
-
-            if flag_overflow.item() > 0:
-                scale_buf = torch.IntTensor([int(scaler._loss_scale)]).cuda()
-                _allreduce_min(scale_buf)
-                scaler._loss_scale = scale_buf.item()
-                scaler._unskipped = 0
-                return True
+    def update_scale_on_all_ranks():
+        overflowed_here = own_update()
+        flag = torch.tensor([1 if overflowed_here else 0], dtype=torch.int32).cuda()
+        _allreduce_sum(flag)
+        if flag.item() == 0:
             return False
-        return wrapper
+        smallest = torch.tensor([int(scaler._loss_scale)], dtype=torch.int32).cuda()
+        _allreduce_min(smallest)
+        scaler._loss_scale = smallest.item()
+        scaler._unskipped = 0
+        return True
 
-    scaler.update_scale = decorate(scaler.update_scale)
+    scaler.update_scale = update_scale_on_all_ranks
     scaler._rannc_patched = True
 
 

@@ -19,9 +19,20 @@ from . import _lib
 from .multi_tensor import dtype_code, stream_handle
 
 
+_data_ptr = torch.Tensor.data_ptr
+_is_contiguous = torch.Tensor.is_contiguous
+
+
+class _Steady:
+    """What a group's last full step established, for the steps after it: as long as the same parameters all
+    have contiguous gradients of the same dtype, a step is one pointer comparison per gradient and one launch."""
+    __slots__ = ("params_obj", "n", "param_ids", "table", "grad_ptrs", "grad_dtype", "steps_buf", "count", "device")
+
+
 class _FusedBase(torch.optim.Optimizer):
     def __init__(self, params, defaults):
         super().__init__(params, defaults)
+        self._steady: Dict[int, _Steady] = {}
         self._tables: Dict[Tuple, Tuple[_lib.OptimTable, Tuple, List]] = {}
         self._model_copies: Dict[int, torch.Tensor] = {}
         self._steps: Dict[int, Tuple[torch.Tensor, int]] = {}     # id(param) -> (its step tensor, value)
@@ -45,6 +56,61 @@ class _FusedBase(torch.optim.Optimizer):
         switch it off."""
         self._grad_sources = {id(p): g for p, g in zip(params, grads) if g is not None}
 
+    def load_state_dict(self, state_dict) -> None:
+        super().load_state_dict(state_dict)
+        self._steady.clear()          # the state tensors are new objects: the next step rebuilds tables and counters
+        self._tables.clear()
+        self._steps.clear()
+
+    def _steady_grads(self, gi: int, group) -> Optional[Tuple["_Steady", List[torch.Tensor]]]:
+        """The group's steady-state record and this step's gradients, or None when anything about the group
+        differs from the step that made the record (then the full path runs and makes a new one)."""
+        st = self._steady.get(gi)
+        params = group["params"]
+        if st is None or st.params_obj is not params or len(params) != st.n:
+            return None
+        if self._grad_sources:
+            grads = list(map(self._grad_sources.get, st.param_ids))
+        else:
+            grads = [p.grad for p in params]
+        for g in grads:
+            if g is None:
+                return None
+        if grads[0].dtype != st.grad_dtype or grads[-1].dtype != st.grad_dtype or not all(map(_is_contiguous, grads)):
+            return None
+        ptrs = list(map(_data_ptr, grads))
+        if ptrs != st.grad_ptrs:
+            st.table.update_pointers(grads=ptrs, stream=stream_handle(st.device))
+            st.grad_ptrs = ptrs
+        return st, grads
+
+    def _make_steady(self, gi: int, group, table, grads: List[torch.Tensor], count: Optional[int]) -> None:
+        params = group["params"]
+        st = _Steady()
+        st.params_obj, st.n = params, len(params)
+        st.param_ids = [id(p) for p in params]
+        st.table = table
+        st.grad_ptrs = [g.data_ptr() for g in grads]
+        st.grad_dtype = grads[0].dtype
+        st.device = params[0].device
+        st.count = count
+        st.steps_buf = None
+        if count is not None:
+            # every parameter's ``step`` becomes a view of one host vector: a step is one add, not one per parameter
+            st.steps_buf = torch.full((len(params),), float(count), dtype=torch.float32)
+            for i, p in enumerate(params):
+                self.state[p]["step"] = st.steps_buf[i]
+                self._steps.pop(id(p), None)      # from here on the tensor itself is the count
+        self._steady[gi] = st
+
+    def zero_grad(self, set_to_none: bool = True) -> None:
+        """``torch.optim.Optimizer.zero_grad`` without its per-parameter bookkeeping."""
+        if not set_to_none:
+            return super().zero_grad(set_to_none=False)
+        for group in self.param_groups:
+            for p in group["params"]:
+                p.grad = None
+
     def _grad_of(self, p: torch.Tensor) -> Optional[torch.Tensor]:
         return self._grad_sources.get(id(p), p.grad) if self._grad_sources else p.grad
 
@@ -59,6 +125,7 @@ class _FusedBase(torch.optim.Optimizer):
             dtype_code(c.dtype)
             self._model_copies[id(m)] = c
         self._tables.clear()
+        self._steady.clear()
 
     def _check_param(self, p: torch.Tensor, g: torch.Tensor) -> None:
         if p.dtype != torch.float32:
@@ -91,8 +158,10 @@ class _FusedBase(torch.optim.Optimizer):
             if old != ptrs:
                 table.update_pointers(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[4] if any(ptrs[4]) else None,
                                       stream_handle(dev))
-        # the table borrows raw pointers: keep what it points at alive
-        self._tables[key] = (table, ptrs, [params, grads, state1, state2, copies])
+        # the table borrows raw pointers: keep what it points at alive - except the gradients, which only have to
+        # live until the launch that reads them is queued (their memory is reused in stream order) and whose
+        # release lets the next backward find the same addresses free
+        self._tables[key] = (table, ptrs, [params, state1, state2, copies])
         return table
 
 
@@ -113,6 +182,17 @@ class FusedAdam(_FusedBase):
             with torch.enable_grad():
                 loss = closure()
         for gi, group in enumerate(self.param_groups):
+            steady = self._steady_grads(gi, group)
+            if steady is not None:
+                st, _ = steady
+                st.count += 1
+                st.steps_buf += 1
+                b1, b2 = group["betas"]
+                st.table.adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], st.count,
+                                   decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
+                                   gate=self.gate, stream=stream_handle(st.device))
+                continue
+            self._steady.pop(gi, None)
             by_step: Dict[int, List[torch.Tensor]] = {}
             step_tensors = []
             grad_of: Dict[int, torch.Tensor] = {}
@@ -145,6 +225,8 @@ class FusedAdam(_FusedBase):
                 table.adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], step,
                                 decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
                                 gate=self.gate, stream=stream_handle(ps[0].device))
+                if len(by_step) == 1 and len(ps) == len(group["params"]):
+                    self._make_steady(gi, group, table, [grad_of[id(p)] for p in ps], step)
         return loss
 
 
@@ -176,6 +258,14 @@ class FusedSGD(_FusedBase):
             with torch.enable_grad():
                 loss = closure()
         for gi, group in enumerate(self.param_groups):
+            steady = self._steady_grads(gi, group)
+            if steady is not None:
+                st, _ = steady
+                st.table.sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
+                                  group["nesterov"], group["maximize"], first_step=False, grad_scale=self.grad_scale,
+                                  gate=self.gate, stream=stream_handle(st.device))
+                continue
+            self._steady.pop(gi, None)
             fresh, seasoned = [], []
             grad_of: Dict[int, torch.Tensor] = {}
             for p in group["params"]:
@@ -200,4 +290,6 @@ class FusedSGD(_FusedBase):
                 table.sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
                                group["nesterov"], group["maximize"], first_step=first, grad_scale=self.grad_scale,
                                gate=self.gate, stream=stream_handle(ps[0].device))
+                if not first and not fresh and len(ps) == len(group["params"]):
+                    self._make_steady(gi, group, table, [grad_of[id(p)] for p in ps], None)
         return loss

@@ -119,6 +119,13 @@ class TensorPlan:
         if dsts is not None:
             self._dsts = list(dsts)
 
+    def repoint_sources(self, src_ptrs: Sequence[int]) -> None:
+        """New source addresses (one per tensor, same sizes and dtypes, contiguous) without any per-tensor check:
+        for callers that have established those facts themselves."""
+        if len(src_ptrs) != self.n:
+            raise ValueError(f"expected {self.n} source addresses")
+        self.plan.update_pointers(src_ptrs, None, self._stream())
+
     def drop_sources(self) -> None:
         """Stop keeping the source tensors alive (the table still points at their memory).  For callers
         that have queued every kernel reading them and will ``update`` the table before its next use;

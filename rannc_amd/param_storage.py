@@ -36,6 +36,25 @@ class _PlanCache:
     def __init__(self) -> None:
         self._key: Optional[tuple] = None
         self._plan: Optional[TensorPlan] = None
+        self._token = None
+        self._src_ptrs: Optional[List[int]] = None
+
+    def get_same_shapes(self, token, srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) -> TensorPlan:
+        """``get`` for a caller that vouches, by passing the same ``token`` as last time, that the list has the
+        sizes, dtypes and destinations it had then (the same parameters, all with gradients): only the source
+        addresses are looked at - one ``data_ptr`` per tensor instead of a signature per pair."""
+        if self._plan is None or token is None or token != self._token or not all(map(torch.Tensor.is_contiguous, srcs)):
+            plan = self.get(srcs, dsts)
+            self._token = token
+            self._src_ptrs = list(map(torch.Tensor.data_ptr, srcs))
+            return plan
+        ptrs = list(map(torch.Tensor.data_ptr, srcs))
+        if ptrs != self._src_ptrs:
+            self._plan.repoint_sources(ptrs)
+            self._src_ptrs = ptrs
+            self._key = None                  # the general signature no longer describes the table
+        self._plan._srcs = list(srcs)
+        return self._plan
 
     def get(self, srcs: Sequence[Optional[torch.Tensor]], dsts: Optional[Sequence[Optional[torch.Tensor]]]) -> TensorPlan:
         def sig(ts):
@@ -44,6 +63,7 @@ class _PlanCache:
             return tuple((0 if t is None else t.data_ptr(), 0 if t is None else t.numel(),
                           None if t is None else t.dtype) for t in ts)
         key = (sig(srcs), sig(dsts))
+        self._token = None
         if self._plan is not None and key == self._key:
             return self._plan
         if self._plan is not None:
@@ -64,7 +84,7 @@ class _PlanCache:
     def clear(self) -> None:
         if self._plan is not None:
             self._plan.close()
-        self._plan, self._key = None, None
+        self._plan, self._key, self._token, self._src_ptrs = None, None, None, None
 
 
 class GradConsolidation:
@@ -263,6 +283,7 @@ class ParamStorage:
         self.consolidate = False
         self.use_amp_master_params: Dict[str, bool] = {}
         self.allreduce_amp_master_params = False
+        self._sorted_ids: Dict[str, List[int]] = {}
         self._clip_plans: Dict[Tuple[str, bool], _PlanCache] = {}
         self._zero_plans: Dict[str, _PlanCache] = {}
         self._scale_plans: Dict[Tuple[str, bool], _PlanCache] = {}
@@ -293,9 +314,13 @@ class ParamStorage:
         return self.graph_params[graph_id]
 
     def sorted_param_ids(self, graph_id: str) -> List[int]:
-        """``getSortedParamIDs`` (``src/comp/ParamStorage.cpp:23-31``): ids in name order."""
-        m = self.graph_params[graph_id]
-        return [m[name] for name in sorted(m)]
+        """``getSortedParamIDs`` (``src/comp/ParamStorage.cpp:23-31``): ids in name order (sorted once per
+        deployment: the per-step operations all walk this list)."""
+        cached = self._sorted_ids.get(graph_id)
+        if cached is None:
+            m = self.graph_params[graph_id]
+            cached = self._sorted_ids[graph_id] = [m[name] for name in sorted(m)]
+        return cached
 
     def zero_enabled(self, graph_id: str) -> bool:
         return graph_id in self.zero_grad_locators
@@ -307,6 +332,7 @@ class ParamStorage:
         """The slice of ``ParamStorage::deploy`` (``src/comp/ParamStorage.cpp:827-1022``) that
         prepares the per-step path: name-sorted id list, ZeRO locator, gradient buckets."""
         self.graph_params[graph_id] = dict(graph_params)
+        self._sorted_ids.pop(graph_id, None)
         self.consolidate = consolidate
         self.use_amp_master_params[graph_id] = use_amp_master_params
         self.allreduce_amp_master_params = allreduce_amp_master_params
@@ -323,6 +349,7 @@ class ParamStorage:
 
     def undeploy(self, graph_id: str) -> None:
         self.graph_params.pop(graph_id, None)
+        self._sorted_ids.pop(graph_id, None)
         self.grad_cons.pop(graph_id, None)
         self.zero_grad_locators.pop(graph_id, None)
         for d in (self._clip_plans, self._scale_plans):
@@ -478,6 +505,18 @@ class ParamStorage:
             if srcs:
                 with torch.no_grad():
                     TensorPlan(srcs, dsts).scale_cast(1.0)
+
+    def gather_tensor_zero(self, ten: torch.Tensor, pid: int) -> torch.Tensor:
+        """``gatherTensorZero`` (``src/comp/ParamStorage.cpp:670-685``) with one rank: the only piece is the
+        whole flattened tensor; it comes back in the parameter's shape
+        (``DistributedParamLocatorBase::gather``, ``src/comp/DistributedParamLocatorBase.cpp:149-152``)."""
+        for graph_id, loc in self.zero_grad_locators.items():
+            if loc.registered(pid) and pid in self.graph_params.get(graph_id, {}).values():
+                param = loc.params[pid]
+                if ten.numel() != param.numel():
+                    raise ValueError(f"tensor has {ten.numel()} elements, parameter {pid} has {param.numel()}")
+                return ten.detach().reshape(param.shape)
+        raise ValueError(f"Param is not registered for zero: {pid}")
 
     def get_local_param_range(self, graph_id: str, pid: int) -> Tuple[int, int]:
         return self.zero_grad_locators[graph_id].get_segment_range(pid)
