@@ -207,8 +207,9 @@ class RaNNCModule(_pyrannc.RaNNCModule):
         if amp_master_param and stash is not None and stash.pending_finish:
             from .amp import finish_unscale
             finish_unscale(self.optimizer)        # the master gradients are about to be looked at: write them
-        p = self.get_param(name, amp_master_param)
-        return p.grad
+        if name not in self.name_to_pid:
+            raise RuntimeError(f"Parameter not found: {name}")       # pyrannc/__init__.py:480-481
+        return super().get_param_grad(self.name_to_pid[name], amp_master_param)
 
     # ------------------------------------------------------------------ checkpoints
     def state_dict(self, *args, no_hook=False, amp_master_params=True, rank0_only=True, **kwargs):

@@ -206,11 +206,31 @@ class RaNNCModule:
         self._check()
         return _param_storage.get_local_param_segment(self.graph_id, param_id)
 
-    def get_param(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
-        self._check()
+    def _owned_tensor(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
         if amp_master_param and _param_storage.has_amp_master_param(param_id):
             return _param_storage.get_amp_master_param_tensor(param_id)
         return _param_storage.get_param_tensor(param_id)
+
+    def _in_param_shape(self, ten: torch.Tensor, param_id: int) -> torch.Tensor:
+        """Under ZeRO the tensor this process steps on is a flat local segment; the reference hands callers
+        the gathered tensor in the parameter's shape (``ParamStorage::doGatherParam`` ->
+        ``gatherTensorZero``, ``src/comp/ParamStorage.cpp:1201-1232, 670-685``)."""
+        shape = _param_storage.get_param_tensor(param_id).shape
+        if ten.shape != shape and ten.numel() == shape.numel():
+            return ten.detach().view(shape)
+        return ten
+
+    def get_param(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
+        self._check()
+        return self._in_param_shape(self._owned_tensor(param_id, amp_master_param), param_id)
+
+    def get_param_grad(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
+        """``gatherParamGrad`` (``src/comp/ParamStorage.cpp:1197-1213``): the gradient of the tensor this
+        process steps on, zeros when it has none, in the parameter's shape."""
+        self._check()
+        owner = self._owned_tensor(param_id, amp_master_param)
+        grad = owner.grad if owner.grad is not None else torch.zeros_like(owner)
+        return self._in_param_shape(grad, param_id)
 
     def undeploy(self) -> None:
         if self._deployed:
