@@ -343,12 +343,13 @@ def run_c5(z: ZeroFlat, op: str, steps: int, warmup: int) -> dict:
     src, dst, bpe = {"c5_unflatten": (z.flat_views, z.params, 4), "c5_master_cast": (z.params, z.masters, 6),
                      "c5_copy_back": (z.masters, z.params, 6), "c5_repack": (z.params, z.flat_views, 4)}[op]
     plan = TensorPlan(src, dst)
+    order = plan.tune()                       # as a caller does once per plan: measured block -> XCD order
     wall, dev_s = timed(lambda: plan.scale_cast(1.0), steps, warmup, 5)
     plan.close()
     nbytes = bpe * z.n
     return entry("c5_zero_flat", op, wall, nbytes,
                  roofline("pass_kernel<write, streaming>", nbytes, dev_s, measured_traffic(op, "c5_zero_flat", "pass_kernel<write>")),
-                 steps=steps, elements=z.n, segments=len(z.sizes))
+                 steps=steps, elements=z.n, segments=len(z.sizes), tuned_write_order=order)
 
 
 # ----------------------------------------------------------------------------- CPU baseline

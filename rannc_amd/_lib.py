@@ -55,6 +55,8 @@ SIGNATURES = {
     "rg_plan_chunk_elems": (_i64, [_vp]),
     "rg_plan_total_numel": (_i64, [_vp]),
     "rg_plan_set_streaming": (_i, [_vp, _i]),
+    "rg_plan_tune": (_i, [_vp, _vp]),
+    "rg_plan_write_order": (_i, [_vp]),
     "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
     "rg_step_begin": (_i, [_vp, _f, _vp]),
     "rg_step_finish": (_i, [_vp, _f, _i, _vp]),
@@ -195,6 +197,12 @@ class Plan:
     def set_streaming(self, mode: int) -> None:
         """1 = nontemporal accesses, 0 = plain, -1 = decide from the plan's size."""
         check(lib.rg_plan_set_streaming(self._handle, mode))
+
+    def tune(self, stream: int = 0) -> int:
+        """Measure the block -> XCD orders on the plan's own tensors and keep the fastest (overwrites the
+        destinations, waits for the stream).  Returns the order chosen."""
+        check(lib.rg_plan_tune(self._handle, _vp(stream)))
+        return int(lib.rg_plan_write_order(self._handle))
 
     def update_pointers(self, src_ptrs: Optional[Sequence[Optional[int]]],
                         dst_ptrs: Optional[Sequence[Optional[int]]], stream: int = 0) -> None:

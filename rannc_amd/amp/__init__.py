@@ -114,10 +114,11 @@ class LossScaler:
         if stash.unscale_cache is None:
             from ..param_storage import _PlanCache
             stash.unscale_cache = _PlanCache()
+        # a new table is tuned on the spot, unless the master gradients hold values that are about to be added to
         if all_params:
-            stash.unscale_plan = stash.unscale_cache.get_same_shapes("all", model_grads, master_grads)
+            stash.unscale_plan = stash.unscale_cache.get_same_shapes("all", model_grads, master_grads, tune_new=not accumulate)
         else:
-            stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads)
+            stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads, tune_new=not accumulate)
         inv = 1.0 / self._loss_scale
         if stash.clip_decided:
             # what the last step decided (still in the table's result block) picks this step's strategy

@@ -10,6 +10,7 @@
 
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "ranncgrad.h"
@@ -133,6 +134,7 @@ class Plan {
     return reinterpret_cast<uintptr_t>(r);
   }
   void unscale_pack(float inv_scale) { check(rg_unscale_pack(handle(), inv_scale, current_stream(device_))); }
+  void step_apply_clip(float max_norm, int flags) { check(rg_step_apply_clip(handle(), max_norm, flags, current_stream(device_))); }
   void accumulate(float scale) { check(rg_accumulate(handle(), scale, current_stream(device_))); }
   void unscale_accumulate(float inv_scale) {
     check(rg_unscale_accumulate(handle(), inv_scale, current_stream(device_)));
@@ -264,6 +266,98 @@ void copy_cast(const py::handle& dst, const py::handle& src, float scale) {
                              current_stream(d.device)));
 }
 
+// ---------------------------------------------------------------------------------------------
+// The free functions of the reference's extension module that sit on this path, under their own
+// names and with their argument meaning (src/main.cpp:55-59, 78-136, 191-245), for one process:
+// a maintainer can register this module's functions as `_pyrannc`'s.  Tensors are identified by
+// the Python id() of the object (src/bind/PybindUtil.cpp:8-12); the registries hold the tensors.
+
+long object_id(const py::handle& o) { return (long)reinterpret_cast<intptr_t>(o.ptr()); }
+
+py::object torch_empty(int64_t n, const py::object& dtype, const py::object& device) {
+  return py::module_::import("torch").attr("empty")(n, py::arg("dtype") = dtype, py::arg("device") = device);
+}
+
+// DistributedParamLocator (src/comp/DistributedParamLocator.cpp:14-83) + gather
+// (src/comp/DistributedParamLocatorBase.cpp:96-153) for a world of one rank.
+class DistParamRegistry {
+ public:
+  struct Entry {
+    int64_t numel = 0, aligned = 0, segment = 0, offset = 0, src_size = 0;
+    py::object shape;       // torch.Size of the full tensor
+    bool requires_grad = false;
+    py::object part;        // this rank's segment
+  };
+
+  py::object store(const py::object& param) {
+    const long pid = object_id(param);
+    Entry e;
+    e.numel = param.attr("numel")().cast<int64_t>();
+    const int esz = param.attr("element_size")().cast<int>();
+    dtype_code(param);                                            // float32 / float16 / bfloat16 only
+    check(rg_segment_layout(e.numel, esz, 1, &e.aligned, &e.segment, &e.offset, &e.src_size));
+    e.shape = param.attr("shape");
+    e.requires_grad = param.attr("requires_grad").cast<bool>();
+    py::object flat = param.attr("detach")().attr("contiguous")().attr("view")(-1).attr("narrow")(0, e.offset, e.src_size);
+    if (param.attr("is_cuda").cast<bool>()) {
+      e.part = torch_empty(e.src_size, param.attr("dtype"), param.attr("device"));
+      if (e.src_size > 0) copy_cast(e.part, flat, 1.0f);
+    } else {
+      // built on the host: the slice is uploaded (a transfer, no arithmetic); the segment lives on the GPU
+      e.part = flat.attr("to")("cuda");
+    }
+    e.part.attr("requires_grad_")(e.requires_grad);
+    entries_[pid] = e;
+    return e.part;
+  }
+  Entry& at(long pid) {
+    auto it = entries_.find(pid);
+    if (it == entries_.end()) throw std::invalid_argument("Parameter is not registered: " + std::to_string(pid));
+    return it->second;
+  }
+  py::object load(long pid) {
+    Entry& e = at(pid);
+    py::object buf = torch_empty(e.segment, e.part.attr("dtype"), e.part.attr("device"));
+    const int64_t n = e.part.attr("numel")().cast<int64_t>();
+    if (n > 0) copy_cast(buf.attr("narrow")(0, 0, n), e.part.attr("detach")(), 1.0f);
+    if (e.segment > n) copy_cast(buf.attr("narrow")(0, n, e.segment - n), py::none(), 1.0f);      // zero padding
+    py::object out = buf.attr("narrow")(0, 0, e.numel).attr("view")(e.shape).attr("cpu")().attr("detach")();
+    out.attr("requires_grad_")(e.requires_grad);
+    return out;
+  }
+  void set(long pid, const py::object& full) {
+    Entry& e = at(pid);
+    if (e.src_size == 0) return;
+    py::object src = full.attr("detach")().attr("to")(e.part.attr("device")).attr("contiguous")().attr("view")(-1)
+                         .attr("narrow")(0, e.offset, e.src_size);
+    copy_cast(e.part.attr("detach")(), src, 1.0f);
+  }
+  void set_dtype(long pid, const py::object& dtype) {
+    Entry& e = at(pid);
+    if (py::object(e.part.attr("dtype")).equal(dtype)) return;
+    py::object fresh = torch_empty(e.part.attr("numel")().cast<int64_t>(), dtype, e.part.attr("device"));
+    dtype_code(fresh);
+    copy_cast(fresh, e.part.attr("detach")(), 1.0f);
+    fresh.attr("requires_grad_")(e.requires_grad);
+    e.part = fresh;
+  }
+  bool registered(long pid) const { return entries_.count(pid) != 0; }
+  void remove(long pid) { entries_.erase(pid); }
+  void clear() { entries_.clear(); }
+
+ private:
+  std::unordered_map<long, Entry> entries_;
+};
+
+DistParamRegistry& dist_params() {
+  static DistParamRegistry* r = new DistParamRegistry();   // never destroyed: it holds Python objects
+  return *r;
+}
+std::unordered_map<long, py::object>& amp_masters() {
+  static auto* m = new std::unordered_map<long, py::object>();
+  return *m;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_ranncgrad, m) {
@@ -274,6 +368,7 @@ PYBIND11_MODULE(_ranncgrad, m) {
   m.attr("STEP_DEFAULT") = (int)RG_STEP_DEFAULT;
   m.attr("STEP_WRITE_ON_OVERFLOW") = (int)RG_STEP_WRITE_ON_OVERFLOW;
   m.attr("STEP_IGNORE_OVERFLOW") = (int)RG_STEP_IGNORE_OVERFLOW;
+  m.attr("STEP_EXPECT_NO_CLIP") = (int)RG_STEP_EXPECT_NO_CLIP;
   m.def("version", &rg_version);
   m.def("aligned_numel", [](int64_t numel, int elem_size, int split) {
     const int64_t r = rg_aligned_numel(numel, elem_size, split);
@@ -289,6 +384,44 @@ PYBIND11_MODULE(_ranncgrad, m) {
   });
   m.def("copy_cast", &copy_cast, py::arg("dst"), py::arg("src"), py::arg("scale") = 1.0f,
         "dst.copy_(src) with dtype conversion and optional scale for one pair of tensors; src=None stores zeros");
+  // -- the reference's names (one process, one GPU)
+  m.def("get_rank", [] { return 0; });
+  m.def("get_world_size", [] { return 1; });
+  m.def("barrier", [] {});
+  m.def("allreduce_tensor", [](const py::object& tensor, bool sum) {
+    (void)sum;                                       // a sum or a minimum over one rank leaves the tensor as it is
+    if (!py::hasattr(tensor, "data_ptr")) throw std::invalid_argument("allreduce_tensor expects a tensor");
+  }, py::arg("tensor"), py::arg("sum"));
+  m.def("bcast_tensor", [](const py::object& tensor, int root) {
+    if (root != 0) throw std::invalid_argument("root " + std::to_string(root) + " is not a rank of this world (size 1)");
+    return tensor.attr("cuda")();
+  });
+  m.def("all_gather", [](const py::object& ten, const py::object& buf) {
+    if (buf.attr("numel")().cast<int64_t>() != ten.attr("numel")().cast<int64_t>())
+      throw std::invalid_argument("all_gather: receive buffer must hold world_size * numel elements");
+    copy_cast(buf.attr("view")(-1), ten.attr("contiguous")().attr("view")(-1), 1.0f);
+  });
+  m.def("register_amp_master_param", [](long model_param_id, const py::object& param) { amp_masters()[model_param_id] = param; });
+  m.def("get_amp_master_param", [](long model_param_id) {
+    auto it = amp_masters().find(model_param_id);
+    if (it == amp_masters().end()) throw std::invalid_argument("Amp master parameter not found: " + std::to_string(model_param_id));
+    return it->second;
+  });
+  m.def("store_dist_param", [](const py::object& param) { return dist_params().store(param); });
+  m.def("load_dist_param", [](long pid) { return dist_params().load(pid); });
+  m.def("set_dist_param", [](long pid, const py::object& full) { dist_params().set(pid, full); });
+  m.def("get_dist_param_segment", [](long pid) { return dist_params().at(pid).part; });
+  m.def("set_dist_param_dtype", [](long pid, const py::object& dtype) { dist_params().set_dtype(pid, dtype); });
+  m.def("get_dist_param_range", [](long pid) {
+    const auto& e = dist_params().at(pid);
+    return py::make_tuple(e.offset, e.offset + e.src_size);
+  });
+  m.def("remove_dist_param", [](long pid) { dist_params().remove(pid); });
+  m.def("dist_param_registered", [](long pid) { return dist_params().registered(pid); });
+  m.def("clear", [] {
+    dist_params().clear();
+    amp_masters().clear();
+  });
   py::class_<Plan>(m, "Plan")
       .def(py::init<const py::sequence&, const py::object&, int64_t>(), py::arg("srcs"), py::arg("dsts") = py::none(),
            py::arg("chunk_elems") = 0)
@@ -299,6 +432,7 @@ PYBIND11_MODULE(_ranncgrad, m) {
       .def("step_decide", &Plan::step_decide, py::arg("max_norm"), py::arg("flags") = 0)
       .def("result_device_ptr", &Plan::result_device_ptr)
       .def("unscale_pack", &Plan::unscale_pack)
+      .def("step_apply_clip", &Plan::step_apply_clip, py::arg("max_norm"), py::arg("flags") = 0)
       .def("accumulate", &Plan::accumulate, py::arg("scale") = 1.0f)
       .def("unscale_accumulate", &Plan::unscale_accumulate)
       .def("grad_norm", &Plan::grad_norm)

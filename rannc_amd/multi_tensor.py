@@ -119,6 +119,12 @@ class TensorPlan:
         if dsts is not None:
             self._dsts = list(dsts)
 
+    def tune(self) -> int:
+        """Let the library measure, on these very tensors, which hand-out order of tiles to the XCDs is fastest
+        for the plan's writing passes, and keep it.  Overwrites the destinations with ``cast(src)`` and waits for
+        the stream: call it once, right after building a plan whose destinations hold nothing yet."""
+        return self.plan.tune(self._stream())
+
     def repoint_sources(self, src_ptrs: Sequence[int]) -> None:
         """New source addresses (one per tensor, same sizes and dtypes, contiguous) without any per-tensor check:
         for callers that have established those facts themselves."""

@@ -30,6 +30,25 @@ def _zeros(n: int, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
     return fill_zero_(torch.empty(n, dtype=dtype, device=device))
 
 
+class BufferTensorCache:
+    """Buffers that live across steps, keyed by a caller-chosen name and re-made only when the requested type
+    changes (``BufferTensorCache``, ``src/torch/TorchUtil.cpp:1434-1461``).  Besides saving the allocations it
+    keeps the buffers' addresses fixed, so the device tables that point at them are built once."""
+
+    def __init__(self) -> None:
+        self._bufs: Dict[str, torch.Tensor] = {}
+
+    def get(self, key: str, numel: int, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() != numel or buf.dtype != dtype or buf.device != device:
+            buf = self._bufs[key] = torch.empty(numel, dtype=dtype, device=device)
+        return buf
+
+    def clear(self, prefix: str = "") -> None:
+        for key in [k for k in self._bufs if k.startswith(prefix)]:
+            del self._bufs[key]
+
+
 class _PlanCache:
     """Reuses a device table while the tensors it describes stay where they are."""
 
@@ -39,12 +58,13 @@ class _PlanCache:
         self._token = None
         self._src_ptrs: Optional[List[int]] = None
 
-    def get_same_shapes(self, token, srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) -> TensorPlan:
+    def get_same_shapes(self, token, srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor],
+                        tune_new: bool = False) -> TensorPlan:
         """``get`` for a caller that vouches, by passing the same ``token`` as last time, that the list has the
         sizes, dtypes and destinations it had then (the same parameters, all with gradients): only the source
         addresses are looked at - one ``data_ptr`` per tensor instead of a signature per pair."""
         if self._plan is None or token is None or token != self._token or not all(map(torch.Tensor.is_contiguous, srcs)):
-            plan = self.get(srcs, dsts)
+            plan = self.get(srcs, dsts, tune_new)
             self._token = token
             self._src_ptrs = list(map(torch.Tensor.data_ptr, srcs))
             return plan
@@ -56,7 +76,10 @@ class _PlanCache:
         self._plan._srcs = list(srcs)
         return self._plan
 
-    def get(self, srcs: Sequence[Optional[torch.Tensor]], dsts: Optional[Sequence[Optional[torch.Tensor]]]) -> TensorPlan:
+    def get(self, srcs: Sequence[Optional[torch.Tensor]], dsts: Optional[Sequence[Optional[torch.Tensor]]],
+            tune_new: bool = False) -> TensorPlan:
+        """``tune_new``: a table that has to be built is also tuned (``TensorPlan.tune``: the destinations are
+        overwritten, so only for callers whose destinations hold nothing they still need)."""
         def sig(ts):
             if ts is None:
                 return None
@@ -78,6 +101,8 @@ class _PlanCache:
                 return self._plan
             self._plan.close()
         self._plan = TensorPlan(srcs, dsts)
+        if tune_new and dsts is not None:
+            self._plan.tune()
         self._key = key
         return self._plan
 
@@ -284,6 +309,7 @@ class ParamStorage:
         self.use_amp_master_params: Dict[str, bool] = {}
         self.allreduce_amp_master_params = False
         self._sorted_ids: Dict[str, List[int]] = {}
+        self._staging = BufferTensorCache()
         self._clip_plans: Dict[Tuple[str, bool], _PlanCache] = {}
         self._zero_plans: Dict[str, _PlanCache] = {}
         self._scale_plans: Dict[Tuple[str, bool], _PlanCache] = {}
@@ -359,6 +385,7 @@ class ParamStorage:
             self._zero_plans.pop(graph_id).clear()
         for k in [k for k in self._stage_plans if k.split("/")[0] == graph_id]:
             self._stage_plans.pop(k).clear()
+        self._staging.clear(graph_id + "/")
 
     # ------------------------------------------------------------------ per-step operations
     def prepare_backward(self, graph_id: str) -> None:
@@ -471,14 +498,14 @@ class ParamStorage:
             grad = param.grad
             aligned = _lib.aligned_numel(grad.numel(), grad.element_size(), 1)
             bdt = torch.float32 if (self.allreduce_amp_master_params and param.dtype == torch.float16) else param.dtype
-            buf = torch.empty(aligned, dtype=bdt, device=grad.device)
+            buf = self._staging.get(f"{graph_id}/{pid}", aligned, bdt, grad.device)
             srcs += [grad.view(-1), None]
             dsts += [buf.narrow(0, 0, grad.numel()), buf.narrow(0, grad.numel(), aligned - grad.numel())]
             back_src.append(buf.narrow(0, 0, grad.numel()))
             back_dst.append(grad.view(-1))
             bufs.append(buf)
         if srcs:
-            # the caching allocator usually hands back last step's addresses: the tables are reused
+            # the staging buffers persist (BufferTensorCache), so the tables are built once
             with torch.no_grad():
                 self._stage_plans.setdefault(graph_id + "/pack", _PlanCache()).get(srcs, dsts).scale_cast(1.0)
                 self._stage_plans.setdefault(graph_id + "/back", _PlanCache()).get(back_src, back_dst).scale_cast(1.0)

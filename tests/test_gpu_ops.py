@@ -323,3 +323,34 @@ def test_chunk_boundaries_follow_the_destination_alignment(dst_name):
         out = dst_arena.cpu()
         assert bool((out[dst_off:o] == 0).all()) and bool((out[:dst_off] == 7.0).all()) and bool((out[o:] == 7.0).all())
     plan.close()
+
+
+def test_plan_tune_changes_only_the_time():
+    """rg_plan_tune measures the block -> XCD orders on the plan's tensors; whatever it picks, a pass writes the
+    same bits.  The destinations are overwritten by the measurement itself (cast of the sources)."""
+    g = torch.Generator().manual_seed(33)
+    cpu = [(torch.randn(n, generator=g) * 8).to(torch.float16) for n in (300001, 17, 70001, 4096, 1)]
+    srcs = place_in_arena(cpu, DEV, 1, 3)
+    dsts = [torch.full((t.numel(),), 7.0, dtype=torch.float32, device=DEV) for t in cpu]
+    plan = TensorPlan(srcs, dsts)
+    plan.scale_cast(0.5)
+    before = [d.cpu().clone() for d in dsts]
+    order = plan.tune()
+    assert order in (0, 64, 256, -1)
+    for d, c in zip(dsts, cpu):
+        assert_bits_equal(d.cpu(), c.float(), "what the measurement leaves behind")
+    plan.scale_cast(0.5)
+    for d, b in zip(dsts, before):
+        assert_bits_equal(d.cpu(), b, "same bits under the tuned order")
+    plan.fused_step(0.125, 1.0)
+    res = plan.result()
+    want = oracle.fused_step(cpu, ["f32"] * len(cpu), 0.125, 1.0)
+    assert math.isclose(res.norm, want.norm, rel_tol=1e-6) and res.clipped == 1
+    plan.close()
+    # in place: left alone
+    t = torch.randn(5000, device=DEV)
+    keep = t.clone()
+    p2 = TensorPlan([t], [t])
+    p2.tune()
+    assert torch.equal(t, keep)
+    p2.close()

@@ -113,3 +113,53 @@ def test_optimizer_table_through_pybind_matches_ctypes():
     oa.close()
     with pytest.raises(RuntimeError, match="closed"):
         oa.sgd_step(0.1)
+
+
+def test_reference_entry_point_names_are_exported():
+    """The free functions of the reference's extension on this path (src/main.cpp:55-59, 78-136, 191-245)."""
+    for name in ("get_rank", "get_world_size", "barrier", "allreduce_tensor", "bcast_tensor", "all_gather",
+                 "register_amp_master_param", "store_dist_param", "load_dist_param", "set_dist_param",
+                 "get_dist_param_segment", "set_dist_param_dtype", "get_dist_param_range", "remove_dist_param",
+                 "dist_param_registered"):
+        assert callable(getattr(_ranncgrad, name)), name
+    assert (_ranncgrad.get_rank(), _ranncgrad.get_world_size()) == (0, 1)
+    assert _ranncgrad.dist_param_registered(12345) is False
+    with pytest.raises(ValueError, match="not registered"):
+        _ranncgrad.get_dist_param_range(12345)
+    with pytest.raises(ValueError, match="root"):
+        _ranncgrad.bcast_tensor(torch.zeros(1), 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_dist_param_functions_of_the_compiled_module_match_the_oracle(dtype):
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(9)
+    full = torch.randn(129, 3, generator=g).to(dtype)
+    p = torch.nn.Parameter(full.to(dev))
+    ora = oracle.DistParamOracle(0, 1)
+    want_part = ora.store(1, full)
+    part = _ranncgrad.store_dist_param(p)
+    pid = id(p)
+    try:
+        assert _ranncgrad.dist_param_registered(pid) and part.requires_grad
+        assert_bits_equal(part.detach().cpu(), want_part, "stored segment")
+        assert tuple(_ranncgrad.get_dist_param_range(pid)) == ora.get_range(1)
+        lo, hi = _ranncgrad.get_dist_param_range(pid)
+        assert_bits_equal(part.detach().cpu(), full.flatten()[lo:hi], "segment == full.flatten()[range]")   # test/common.py:57-63
+        loaded = _ranncgrad.load_dist_param(pid)
+        assert not loaded.is_cuda and loaded.shape == full.shape and loaded.requires_grad
+        assert_bits_equal(loaded.detach(), oracle.DistParamOracle.load(1, [ora]), "loaded tensor")
+        new = torch.randn(129, 3, generator=g).to(dtype)
+        _ranncgrad.set_dist_param(pid, new.to(dev))
+        ora.set(1, new)
+        assert_bits_equal(_ranncgrad.get_dist_param_segment(pid).detach().cpu(), ora.parts[1], "set")
+        _ranncgrad.set_dist_param_dtype(pid, torch.float32)
+        ora.set_scalar_type(1, torch.float32)
+        seg = _ranncgrad.get_dist_param_segment(pid)
+        assert seg.dtype == torch.float32 and seg.requires_grad
+        assert_bits_equal(seg.detach().cpu(), ora.parts[1], "cast segment")
+        assert_bits_equal(_ranncgrad.load_dist_param(pid).detach(), new.float(), "loaded after cast")
+    finally:
+        _ranncgrad.remove_dist_param(pid)
+    assert not _ranncgrad.dist_param_registered(pid)
