@@ -48,8 +48,8 @@ def parse_args():
     ap.add_argument("--c5-elements", type=int, default=10_000_000_000, help="total elements of the ZeRO flat buffer")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run three plain 1 GiB fp32 tensor copies first (known traffic, for scaling "
-                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+                    help="also run three plain elementwise kernels over 1 GiB of fp32 first (out = in * 1.5: 1 GiB read, "
+                         "1 GiB written; known traffic for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget for the CPU baseline leg")
     return ap.parse_args()
 
@@ -678,10 +678,12 @@ def main() -> int:
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     if args.calibrate_copy:
+        # one elementwise kernel that reads 1 GiB and writes 1 GiB (a device-to-device copy_ may be split
+        # into several dispatches): the yardstick for what FETCH_SIZE / WRITE_SIZE report per byte moved
         a = torch.empty(256 << 20, dtype=torch.float32, device=dev).fill_(1.0)
         b = torch.empty_like(a)
         for _ in range(3):
-            b.copy_(a)
+            torch.mul(a, 1.5, out=b)
         torch.cuda.synchronize()
         del a, b
         torch.cuda.empty_cache()
