@@ -145,6 +145,9 @@ class StepWorkload:
             off += g.numel()
         self.s, self.d = self.grads[0].element_size(), self.bucket.element_size()
         self.plan = TensorPlan(self.grads, self.views, chunk_elems=chunk_elems)
+        # as a caller does once per plan: the library times its block -> XCD orders on this plan's own tensors
+        # (destinations hold zeros here; a real caller tunes before the first step, when they are dead too)
+        self.write_order = self.plan.tune()
 
     def close(self):
         self.plan.close()
@@ -154,7 +157,8 @@ class StepWorkload:
     def describe(self) -> dict:
         return {"workload": self.key, "description": self.cfg.description, "tensors": len(self.grads), "elements": self.n,
                 "src_bytes_per_elem": self.s, "dst_bytes_per_elem": self.d,
-                "chunk_elems": self.plan.plan.chunk_elems, "chunks": self.plan.plan.num_chunks}
+                "chunk_elems": self.plan.plan.chunk_elems, "chunks": self.plan.plan.num_chunks,
+                "tuned_write_order": self.write_order}
 
 
 def run_fused_step(w: StepWorkload, steps: int, warmup: int, op: str = "fused_step") -> dict:

@@ -97,6 +97,13 @@ constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial st
 // Pass selection for the chunk kernel.
 enum : int { kModeReduce = 1, kModeWrite = 2, kModeAccumulate = 4 };  // accumulate: dst = round(dst + x * scale)
 
+// What one wavefront of a pass that reduces and writes leaves behind: one 16-byte store.
+struct alignas(16) WavePartial {
+  double sumsq;
+  int32_t bad;
+  int32_t pad;
+};
+
 struct PassArgs {
   const ChunkRec* chunks;        // [n_chunks]; null = one tensor described by `single`
   ChunkRec single;               // whole-tensor pointers and types (len unused)
@@ -105,8 +112,9 @@ struct PassArgs {
   int64_t single_head;           // elements before the first aligned chunk boundary
   int32_t xcd_run;               // block -> XCD mapping, see pass_kernel
   int32_t peel_heads;            // writing passes: some destination starts off a boundary
-  double* chunk_sumsq;           // [n_chunks * tiles_per_chunk] written when reducing
-  int32_t* chunk_bad;            // [n_chunks * tiles_per_chunk] written when reducing
+  double* chunk_sumsq;           // [n_chunks] written by a read-only reducing pass
+  int32_t* chunk_bad;            // [n_chunks]
+  WavePartial* wave_partials;    // [blocks * wavefronts per block] written by a pass that reduces and writes
   const StepResult* result;      // non-null: take coef / overflow gate from the device
   int64_t n_chunks;
   int32_t tile_elems;            // elements one block handles (== chunk_elems unless the pass splits chunks)
@@ -136,8 +144,7 @@ struct FinalizeArgs {
 };
 
 struct CombineArgs {
-  const double* tile_sumsq;   // [n_chunks * partials_per_chunk], chunk-major
-  const int32_t* tile_bad;
+  const WavePartial* partials;   // [n_chunks * partials_per_chunk], chunk-major
   double* chunk_sumsq;        // [n_chunks]
   int32_t* chunk_bad;
   int64_t n_chunks;

@@ -258,9 +258,13 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
   constexpr bool kWavePartials = (MODE & kModeReduce) != 0 && (MODE & kModeWrite) != 0;
   constexpr int kSlots = kWavePartials ? T / 64 : 1;
   if (start >= end) {
-    if ((MODE & kModeReduce) && threadIdx.x < kSlots) {
-      a.chunk_sumsq[slot_id * kSlots + threadIdx.x] = 0.0;
-      a.chunk_bad[slot_id * kSlots + threadIdx.x] = 0;
+    if constexpr (kWavePartials) {
+      if (threadIdx.x < kSlots) a.wave_partials[slot_id * kSlots + threadIdx.x] = WavePartial{0.0, 0, 0};
+    } else if (MODE & kModeReduce) {
+      if (threadIdx.x == 0) {
+        a.chunk_sumsq[slot_id] = 0.0;
+        a.chunk_bad[slot_id] = 0;
+      }
     }
     return;
   }
@@ -342,10 +346,8 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
         }
         bad = __any(mine) ? 1 : 0;
       }
-      if ((threadIdx.x & 63) == 0) {
-        a.chunk_sumsq[slot_id * kSlots + (threadIdx.x >> 6)] = s;
-        a.chunk_bad[slot_id * kSlots + (threadIdx.x >> 6)] = bad;
-      }
+      // sum and flag leave in one 16-byte store
+      if ((threadIdx.x & 63) == 0) a.wave_partials[slot_id * kSlots + (threadIdx.x >> 6)] = WavePartial{s, bad, 0};
     } else {
       // One partial per block, the wavefronts combined through LDS in index order.
       __shared__ double wave_sum[kWaves];
@@ -395,13 +397,13 @@ __global__ __launch_bounds__(kBlockThreads) void combine_tiles_kernel(CombineArg
   const int64_t c = (int64_t)blockIdx.x * (kBlockThreads / 64) + (threadIdx.x >> 6);
   if (c >= a.n_chunks) return;
   const int lane = threadIdx.x & 63;
-  const double* ps = a.tile_sumsq + c * a.partials_per_chunk;
-  const int32_t* pb = a.tile_bad + c * a.partials_per_chunk;
+  const WavePartial* ps = a.partials + c * a.partials_per_chunk;
   double s = 0.0;
   int bad = 0;
   for (int i = lane; i < a.partials_per_chunk; i += 64) {
-    s += ps[i];
-    bad |= pb[i];
+    const WavePartial w = ps[i];
+    s += w.sumsq;
+    bad |= w.bad;
   }
   s = wave_total(s);
   bad = __any(bad) ? 1 : 0;
