@@ -661,6 +661,7 @@ def run_one(args, key: str, op: str, steps: int, warmup: int) -> tuple:
         e = run_overflow_host_gate(w, steps, warmup)
     else:
         e = run_plan_op(w, op, steps, warmup)
+    e.setdefault("tuned_write_order", w.write_order)
     desc = w.describe()
     dtype = f"{w.cfg.grad_dtype}->{w.cfg.bucket_dtype} (fp32 arithmetic)"
     w.close()
