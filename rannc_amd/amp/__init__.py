@@ -13,8 +13,10 @@ Two layers live here:
   copy after a step.  Attribute names follow Apex (``_amp_state.loss_scalers``,
   ``optimizer._amp_stash.all_fp16_params`` ...) because the reference reads them.
 
-The dynamic loss-scale schedule (halve on overflow, double after ``scale_window`` clean
-steps) is this project's own statement of the usual policy; Apex's is not in the tree.
+The dynamic loss-scale schedule is Apex's published ``LossScaler.update_scale`` (halve on
+overflow with an optional floor, zero the clean-step counter; otherwise count the step and
+double, up to ``max_loss_scale``, every ``scale_window`` clean steps; a static scale never
+skips), restated here because Apex itself is not in the reference tree.
 
 Gradient accumulation follows PyTorch's convention: a master gradient that is still defined
 when a ``scale_loss`` context exits (no ``zero_grad`` since the last one) is accumulated into
