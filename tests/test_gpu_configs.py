@@ -63,6 +63,33 @@ def test_config_against_oracle(key, scale):
     plan.close()
 
 
+def test_c1_pack_then_unflatten_back():
+    """Configuration 1 end to end: the eight MLP gradients packed into one fp32 bucket by the fused step, then the
+    bucket unflattened back into one separately allocated tensor per parameter - each must hold exactly the slice
+    of the oracle's bucket that belongs to it."""
+    cfg = step_config("c1_mlp")
+    grads_cpu, _ = make_grads(cfg, seed=0, device="cpu")
+    ddt = TORCH_DTYPE[cfg.bucket_dtype]
+    dev = [g.to(DEV) for g in grads_cpu]
+    bucket, views = _bucket_views(dev, ddt)
+    pack = TensorPlan(dev, views)
+    pack.fused_step(cfg.inv_scale, cfg.max_norm)
+    res = pack.result()
+    outs = [torch.full(g.shape, 7.0, dtype=ddt, device=DEV) for g in dev]
+    back = TensorPlan(views, outs)
+    back.scale_cast(1.0)
+    want = oracle.fused_step(grads_cpu, [cfg.bucket_dtype] * len(grads_cpu), cfg.inv_scale, math.inf).buckets[cfg.bucket_dtype]
+    want.mul_(float(res.coef))
+    off = 0
+    for g, o in zip(grads_cpu, outs):
+        assert o.shape == g.shape
+        assert_bits_equal(o.cpu().view(-1), want.narrow(0, off, g.numel()), "unflattened")
+        off += g.numel()
+    assert off == want.numel()
+    pack.close()
+    back.close()
+
+
 def _full_size_check(key):
     cfg = step_config(key)
     grads, injected = make_grads(cfg, seed=0, device=DEV)

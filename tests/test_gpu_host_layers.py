@@ -147,6 +147,40 @@ def test_scale_and_unscale_grads():
     assert all(bool((p.grad == 3.0).all()) for p in ps)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("world", [3, 8])
+def test_scale_and_unscale_grads_random_values(dtype, world):
+    """``doScaleGrads`` (``src/comp/ParamStorage.cpp:598-615``) on random gradients of odd sizes, one of them
+    missing: ``grad.mul_(ratio)`` / ``grad.mul_(1 / ratio)`` with ``ratio = 1 / world`` in double, i.e. ATen's
+    multiply by ``float(ratio)`` rounded to the gradient's dtype - checked bit for bit against torch on the CPU."""
+    gen = torch.Generator().manual_seed(11)
+    shapes = [(257, 3), (1,), (4099,), (64, 65)]
+    ps = _params(shapes, [dtype] * len(shapes))
+    st = ParamStorage()
+    ids, host = {}, []
+    for i, p in enumerate(ps):
+        st.register_param(id(p), p)
+        ids[f"p{i}"] = id(p)
+        if i == 1:
+            host.append(None)          # no gradient: left alone
+            continue
+        g = (torch.randn(p.shape, generator=gen) * 3.0).to(dtype)
+        host.append(g.clone())
+        p.grad = g.to(p.device)
+    st.deploy("g", ids)
+    ratio = 1.0 / float(world)
+    st.scale_grads("g", False, world_size=world)
+    want = [None if g is None else g.clone().mul_(ratio) for g in host]
+    for p, w in zip(ps, want):
+        assert (p.grad is None) == (w is None)
+        if w is not None:
+            assert_bits_equal(p.grad.cpu(), w, "scaled")
+    st.unscale_grads("g", False, world_size=world)
+    for p, w in zip(ps, want):
+        if w is not None:
+            assert_bits_equal(p.grad.cpu(), w.clone().mul_(1.0 / ratio), "unscaled")
+
+
 # ----------------------------------------------------------------------------- ZeRO views
 
 def test_zero_locator_views_and_staging():
