@@ -661,7 +661,8 @@ def run_one(args, key: str, op: str, steps: int, warmup: int) -> tuple:
         e = run_overflow_host_gate(w, steps, warmup)
     else:
         e = run_plan_op(w, op, steps, warmup)
-    e.setdefault("tuned_write_order", w.write_order)
+    if op not in ("copy_back", "unflatten_back"):
+        e.setdefault("tuned_write_order", w.write_order)
     desc = w.describe()
     dtype = f"{w.cfg.grad_dtype}->{w.cfg.bucket_dtype} (fp32 arithmetic)"
     w.close()
@@ -733,6 +734,8 @@ def main() -> int:
                 configs.append(run_overflow_host_gate(w, st, args.warmup))
             else:
                 configs.append(run_plan_op(w, op2, st, args.warmup))
+            if op2 not in ("copy_back", "unflatten_back"):      # those run on a plan of their own, not tuned
+                configs[-1].setdefault("tuned_write_order", w.write_order)
         if w is not None:
             w.close()
         free, _ = torch.cuda.mem_get_info()

@@ -22,6 +22,10 @@
 // MFMA.  LDS is used only for the 4-wavefront combine of the partial sums.
 #include <type_traits>
 
+// the passes of this file write one stream per launch: see the note on streaming stores in rg_device.h
+#ifndef RG_STREAM_STORE_BITS
+#define RG_STREAM_STORE_BITS "sc1 nt"
+#endif
 #include "rg_device.h"
 #include "rg_internal.h"
 
