@@ -125,6 +125,7 @@ struct PassArgs {
   int32_t norm_of_source;        // reduce pass: measure the source as stored (no rounding to dst)
   int32_t only_if_clipped;       // with `result`: the whole launch does nothing unless result->clipped is set
   int32_t src_is_dst;            // read the destination instead of the record's source (in-place rescale)
+  int32_t chunks_per_block;      // launch_gated_pass only: consecutive chunks one block walks through
 };
 
 struct FinalizeArgs {
@@ -153,6 +154,8 @@ struct CombineArgs {
 
 // streaming: nontemporal loads/stores (data far larger than the caches).
 hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream);
+// A whole-chunk write pass that runs only if result->clipped is set, launched with few blocks.
+hipError_t launch_gated_pass(const PassArgs& a, bool streaming, hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream);
 hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream);
 hipError_t launch_combine_tiles(const CombineArgs& a, hipStream_t stream);

@@ -199,39 +199,16 @@ __device__ __forceinline__ int rescan_nonfinite(const char* sp, int len) {
   return bad;
 }
 
+// What one block does with block index `bid` of a pass (after any block -> XCD remapping):
+// tile (bid % tiles_per_chunk) of chunk (bid / tiles_per_chunk).
 // PEEL (writing passes only): some tensor's destination starts off a 128-byte boundary, so
 // blocks look for an unaligned head.  Plans whose destinations are all aligned run the
 // variant compiled without that logic (about 1 % faster on BERT-large).
 template <int MODE, bool NT, bool PEEL>
-__global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs a) {
-  // Block -> (chunk, tile of the chunk); its partial sum, if any, goes to slot blockIdx.x.
+__device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, float coef) {
   constexpr int T = PassThreads<MODE>::value;
-  unsigned bid = blockIdx.x;
-  if (a.xcd_run != 0) {
-    // Workgroups go to the 8 XCDs round-robin.  xcd_run < 0: each XCD gets one contiguous
-    // eighth of the blocks; xcd_run = R > 0: each XCD gets runs of R consecutive blocks.
-    const unsigned nb = gridDim.x, x = bid & 7u, q = bid >> 3;
-    if (a.xcd_run < 0) {
-      bid = x * (nb >> 3) + (x < (nb & 7u) ? x : (nb & 7u)) + q;
-    } else {
-      const unsigned R = (unsigned)a.xcd_run, group = 8u * R;
-      const unsigned g = bid / group;
-      if ((g + 1) * group <= nb) bid = g * group + x * R + (q % R);   // the ragged last group keeps its order
-    }
-  }
   const int64_t c = (int64_t)(bid / (unsigned)a.tiles_per_chunk);
   const int tile = (int)(bid % (unsigned)a.tiles_per_chunk);
-  float coef = 1.0f;
-  if (a.result != nullptr) {
-    // Values produced by the finalize kernel earlier on the same stream.
-    if (a.only_if_clipped != 0) {
-      if (a.result->clipped == 0) return;
-    } else if (a.result->skipped != 0 && a.write_on_overflow == 0) {
-      return;
-    }
-    coef = a.result->coef;
-  }
-
   ChunkRec rec;
   if (a.chunks != nullptr) {
     rec = a.chunks[c];
@@ -376,6 +353,49 @@ __global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs
       }
     }
   }
+}
+
+template <int MODE, bool NT, bool PEEL>
+__global__ __launch_bounds__(PassThreads<MODE>::value) void pass_kernel(PassArgs a) {
+  // Block -> (chunk, tile of the chunk); its partial sum, if any, goes to the slot of that index.
+  unsigned bid = blockIdx.x;
+  if (a.xcd_run != 0) {
+    // Workgroups go to the 8 XCDs round-robin.  xcd_run < 0: each XCD gets one contiguous
+    // eighth of the blocks; xcd_run = R > 0: each XCD gets runs of R consecutive blocks.
+    const unsigned nb = gridDim.x, x = bid & 7u, q = bid >> 3;
+    if (a.xcd_run < 0) {
+      bid = x * (nb >> 3) + (x < (nb & 7u) ? x : (nb & 7u)) + q;
+    } else {
+      const unsigned R = (unsigned)a.xcd_run, group = 8u * R;
+      const unsigned g = bid / group;
+      if ((g + 1) * group <= nb) bid = g * group + x * R + (q % R);   // the ragged last group keeps its order
+    }
+  }
+  float coef = 1.0f;
+  if (a.result != nullptr) {
+    // Values produced by the finalize kernel earlier on the same stream.
+    if (a.only_if_clipped != 0) {
+      if (a.result->clipped == 0) return;
+    } else if (a.result->skipped != 0 && a.write_on_overflow == 0) {
+      return;
+    }
+    coef = a.result->coef;
+  }
+
+  pass_block<MODE, NT, PEEL>(a, bid, coef);
+}
+
+// A write pass that is expected to find nothing to do (an in-place multiply that only runs when the step
+// clipped): each block takes `chunks_per_block` consecutive chunks, so that the launch has few blocks to
+// retire when the decision says "not clipped".  When it does run it is slower than the tiled pass.
+template <bool NT, bool PEEL>
+__global__ __launch_bounds__(PassThreads<kModeWrite>::value) void gated_pass_kernel(PassArgs a) {
+  if (a.result->clipped == 0) return;
+  const float coef = a.result->coef;
+  const int64_t first = (int64_t)blockIdx.x * a.chunks_per_block;
+  int64_t last = first + a.chunks_per_block;
+  if (last > a.n_chunks) last = a.n_chunks;
+  for (int64_t c = first; c < last; ++c) pass_block<kModeWrite, NT, PEEL>(a, (unsigned)c, coef);
 }
 
 // Fixed-order sum of one value per thread over the block: DPP row scans inside each
@@ -534,6 +554,21 @@ hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t 
       launch_mode<kModeReduce | kModeWrite | kModeAccumulate>(a, streaming, stream);
       break;
     default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_gated_pass(const PassArgs& a, bool streaming, hipStream_t stream) {
+  if (a.n_chunks <= 0) return hipSuccess;
+  if (a.result == nullptr || a.chunks_per_block < 1 || a.tiles_per_chunk != 1) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)((a.n_chunks + a.chunks_per_block - 1) / a.chunks_per_block)), block(PassThreads<kModeWrite>::value);
+  const bool peel = a.peel_heads != 0;
+  if (streaming) {
+    if (peel) hipLaunchKernelGGL((gated_pass_kernel<true, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((gated_pass_kernel<true, false>), grid, block, 0, stream, a);
+  } else {
+    if (peel) hipLaunchKernelGGL((gated_pass_kernel<false, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((gated_pass_kernel<false, false>), grid, block, 0, stream, a);
   }
   return hipGetLastError();
 }

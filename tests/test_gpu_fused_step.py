@@ -255,6 +255,30 @@ def test_expect_no_clip_strategy_matches_the_oracle(src_name, dst_name, max_norm
         assert res.clipped == (1 if max_norm == 0.5 else 0)
 
 
+@pytest.mark.parametrize("in_place", [False, True])
+def test_gated_scale_with_several_chunks_per_block(in_place):
+    """More than 16384 chunks: the in-place multiply behind a one-pass write hands each of its blocks several
+    consecutive chunks.  A step that clips against expectation must still write the bits of the two-pass step,
+    ragged tensor ends and the last, partly filled block of chunks included."""
+    shapes = [(17_000_001,), (1023,), (20_500_003,), (1,), (2_000_000,)]     # 19,000+ chunks of 2048 elements
+    grads = _grads(shapes, torch.float32, 1e-2, 1.0, seed=26)
+    if in_place:
+        dev = place_in_arena(grads, DEV, 1, 1)
+        plan = TensorPlan(dev, dev, chunk_elems=2048)
+        assert plan.plan.num_chunks > 16384 + 3
+        plan.fused_step(1.0, 0.25, _lib.RG_STEP_IGNORE_OVERFLOW | _lib.RG_STEP_EXPECT_NO_CLIP)
+        res = plan.result()
+        assert res.clipped == 1
+        coef = torch.tensor(res.coef, dtype=torch.float32)
+        for g, d in zip(grads, dev):
+            assert_bits_equal(d, g * coef, "clipped in place")
+        plan.close()
+        return
+    res, tn, out = _run_fused(grads, torch.float32, 1.0, 0.25, flags=_lib.RG_STEP_EXPECT_NO_CLIP, chunk_elems=2048)
+    assert res.clipped == 1
+    _check_against_oracle(grads, "f32", 1.0, 0.25, res, tn, out)
+
+
 def test_expect_no_clip_on_overflow_leaves_the_unscaled_values():
     grads = _grads([(5000,), (17,), (40000,)], torch.float16, 1e-2, 64.0, seed=22)
     grads[2].view(-1)[12345] = float("inf")
