@@ -92,6 +92,7 @@ __host__ __device__ inline int head_elems(uintptr_t addr, unsigned align, unsign
 }
 constexpr int64_t kChunkQuantum = 2048;    // chunk sizes are multiples of this many elements
 constexpr int64_t kMaxChunkElems = 1 << 20;
+constexpr unsigned kReducePassLdsBytes = 32768;   // dynamic LDS of the streaming read-only pass: 5 resident blocks per compute unit
 constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan
 
 // Pass selection for the chunk kernel.

@@ -20,6 +20,7 @@
 //
 // The work is purely bandwidth bound (a few ALU ops per element): no LDS staging and no
 // MFMA.  LDS is used only for the 4-wavefront combine of the partial sums.
+#include <cstdlib>
 #include <type_traits>
 
 // the passes of this file write one stream per launch: see the note on streaming stores in rg_device.h
@@ -532,12 +533,19 @@ template <int MODE>
 void launch_mode(const PassArgs& a, bool streaming, hipStream_t stream) {
   const dim3 grid((unsigned)(a.n_chunks * a.tiles_per_chunk)), block(PassThreads<MODE>::value);
   const bool peel = (MODE & kModeWrite) == 0 || a.peel_heads != 0;
+  // Unused dynamic LDS caps the blocks resident per compute unit (160 KiB each).  Measured on MI355X: the
+  // streaming read-only pass is fastest with 4-5 blocks of 256 threads per unit instead of the 8 that fit
+  // (7.1 -> 7.4 TB/s on 2.5e9 fp16 elements); every writing pass wants all the blocks it can get.
+  unsigned lds = (MODE == kModeReduce && streaming) ? kReducePassLdsBytes : 0u;
+#ifdef RG_TUNING_ENV   // experiment builds only
+  if (const char* env = getenv((MODE & kModeWrite) ? "RG_LDS_WRITE" : "RG_LDS_REDUCE")) lds = (unsigned)atoi(env);
+#endif
   if (streaming) {
-    if (peel) hipLaunchKernelGGL((pass_kernel<MODE, true, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((pass_kernel<MODE, true, false>), grid, block, 0, stream, a);
+    if (peel) hipLaunchKernelGGL((pass_kernel<MODE, true, true>), grid, block, lds, stream, a);
+    else hipLaunchKernelGGL((pass_kernel<MODE, true, false>), grid, block, lds, stream, a);
   } else {
-    if (peel) hipLaunchKernelGGL((pass_kernel<MODE, false, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((pass_kernel<MODE, false, false>), grid, block, 0, stream, a);
+    if (peel) hipLaunchKernelGGL((pass_kernel<MODE, false, true>), grid, block, lds, stream, a);
+    else hipLaunchKernelGGL((pass_kernel<MODE, false, false>), grid, block, lds, stream, a);
   }
 }
 

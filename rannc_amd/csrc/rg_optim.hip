@@ -1,3 +1,4 @@
+#include <cstdlib>
 // Multi-tensor optimizer step (Adam / AdamW / SGD) with the fp32 -> fp16/bf16 model copy
 // folded in.  Same launch shape as the writing passes of the gradient path: a device-
 // resident table of chunk records, blocks of 128 threads over 1024-element tiles, four
@@ -450,8 +451,12 @@ static int launch_optim(const rg_optim* o, const OptConst& c, const rg_step_resu
   a.c = c;
   const dim3 grid((unsigned)(o->n_chunks * a.tiles_per_chunk)), block(OptShape<ALGO>::kThreads);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (o->total_numel * bytes_per_elem > ((int64_t)256 << 20)) hipLaunchKernelGGL((optim_kernel<ALGO, true>), grid, block, 0, s, a);
-  else hipLaunchKernelGGL((optim_kernel<ALGO, false>), grid, block, 0, s, a);
+  unsigned lds = 0;
+#ifdef RG_TUNING_ENV   // experiment builds only: unused dynamic LDS caps the blocks resident per compute unit
+  if (const char* env = getenv("RG_LDS_OPTIM")) lds = (unsigned)atoi(env);
+#endif
+  if (o->total_numel * bytes_per_elem > ((int64_t)256 << 20)) hipLaunchKernelGGL((optim_kernel<ALGO, true>), grid, block, lds, s, a);
+  else hipLaunchKernelGGL((optim_kernel<ALGO, false>), grid, block, lds, s, a);
   RG_HIP(hipGetLastError());
   return RG_OK;
 }
