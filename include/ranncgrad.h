@@ -121,8 +121,9 @@ int rg_plan_set_streaming(rg_plan* plan, int mode);
 
 /* Optional: choose the order in which the plan's writing passes hand their tiles to the GPU's eight XCDs by
  * measuring it.  Runs the pass `dst = round_dst(float(src))` (what rg_scale_cast(plan, 1.0) writes) a few times
- * under each order the library knows, on the plan's own tensors and on `stream`, waits for them, and keeps the
- * fastest for every later writing pass of this plan.  The destinations are overwritten, so call it where their
+ * under each order the library knows (three interleaved rounds), on the plan's own tensors and on `stream`, waits
+ * for them, and keeps the fastest for every later writing pass of this plan - the order in use is only given up
+ * for one that is more than 1 % faster.  The destinations are overwritten, so call it where their
  * contents do not matter yet (right after creating the plan); in-place plans are left alone.  Results never
  * depend on the order - only the time does.  No counterpart in the reference (it has no kernels to tune).
  * rg_plan_write_order returns the order in use (0 = round robin, n > 0 = runs of n tiles per XCD, -1 = one
