@@ -746,6 +746,22 @@ def main() -> int:
             z.close()
         else:
             configs.append({"workload": "c5_zero_flat", "skipped": f"needs {args.c5_elements * 8 / 1e9:.0f} GB of device memory"})
+        # the optimizer step behind the clip and the host cost of the drop-in API, one compact row each
+        import argparse
+        for op3 in ("adam", "adam_from_model_grads", "sgd"):
+            sub_args = argparse.Namespace(**dict(vars(args), op=op3, steps=sub, no_cpu_baseline=True))
+            r = bench_optimizer(sub_args, "c2_bert_large", torch, dev)
+            configs.append({"workload": "c2_bert_large", "op": op3, "ms_per_step": r["ms_per_step"], "GB/s": r["value"],
+                            "pct_of_hbm_peak": r["pct_of_hbm_peak"], "bytes_per_elem": r["config"]["bytes_per_elem"],
+                            "roofline": r["roofline"], "steps": sub})
+        for k3 in ("c4_resnet152x2", "c2_bert_large"):
+            sub_args = argparse.Namespace(**dict(vars(args), op="api_step", steps=max(args.steps, 30)))
+            r = bench_api_step(sub_args, k3)
+            configs.append({"workload": k3, "op": "api_step", "what": "scale_loss exit + clip_grad_norm + FusedAdam.step + zero_grad "
+                            "through RaNNCModule / amp, wall time per training step",
+                            "us_per_step": r["value"], "device_us_per_step": r["device_us_per_step"],
+                            "host_only_us_per_step": r["host_us_per_step"], "host_us_per_call": r["host_only"]["us_per_call"],
+                            "tensors": r["config"]["tensors"], "steps": sub_args.steps})
         out["configs"] = configs
 
     if not args.no_cpu_baseline and key != "c5_zero_flat":
