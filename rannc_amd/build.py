@@ -45,6 +45,25 @@ def build_pybind(verbose: bool = True) -> str:
     return out
 
 
+def build_abi_driver(verbose: bool = True) -> str:
+    """Compile tests/abi_driver.c - the C ABI driven from plain C99 with only the HIP runtime beside it - into
+    tests/abi_driver (run by tests/test_gpu_c_abi.py on the GPU)."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    out = os.path.join(ROOT, "tests", "abi_driver")
+    cmd = [os.environ.get("CC", "gcc"), "-std=c99", "-O1", "-Wall", "-Wextra", "-Werror", "-ffp-contract=off",
+           "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(rocm, "include"), "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "abi_driver.c"), "-o", out + ".tmp",
+           "-L", HERE, "-l:" + LIB_NAME, "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-lm",
+           "-Wl,-rpath,$ORIGIN/../rannc_amd", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"C driver build failed ({proc.returncode}):\n{proc.stdout}")
+    os.replace(out + ".tmp", out)
+    return out
+
+
 def build(verbose: bool = True) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     srcs = [os.path.join(HERE, "csrc", s) for s in SOURCES]
@@ -65,4 +84,5 @@ def build(verbose: bool = True) -> str:
 if __name__ == "__main__":
     build()
     build_pybind()
+    build_abi_driver()
     sys.exit(0)

@@ -64,3 +64,15 @@ def test_plan_create_rejects_bad_arguments_before_touching_a_device():
         _lib.Plan(0, [0x1001], [None], [10], [_lib.RG_F16], [_lib.RG_F16])
     with pytest.raises(ValueError, match="numel"):
         _lib.Plan(0, [None], [None], [-1], [0], [0])
+
+
+def test_header_is_plain_c99():
+    """The boundary is a C ABI: the header must compile as C99 (no C++ constructs, no torch or HIP types)."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    proc = subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", HEADER],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout
