@@ -60,8 +60,11 @@ def _place(tensors_by_dtype_order, rng, fill=0.0):
     return out
 
 
+@pytest.mark.parametrize("one_pass", [False, True])
 @pytest.mark.parametrize("seed", range(24))
-def test_random_fused_step(seed):
+def test_random_fused_step(seed, one_pass):
+    """``one_pass``: the same cases under RG_STEP_EXPECT_NO_CLIP (write while summing, in-place multiply only if the
+    step clips after all) - same bits; after an overflow that strategy has written the unscaled values."""
     rng, sizes, pairs, srcs_cpu, inv_scale = _random_case(seed)
     srcs = _place(srcs_cpu, rng)
     dsts = _place([torch.full((n,), 3.0, dtype=dd) for n, (_, dd) in zip(sizes, pairs)], rng, fill=3.0)
@@ -69,7 +72,7 @@ def test_random_fused_step(seed):
     plan_srcs = [None if i in missing else s for i, s in enumerate(srcs)]
     max_norm = rng.choice([1e-3, 0.5, 1e6])
     plan = TensorPlan(plan_srcs, dsts, chunk_elems=rng.choice([0, 2048, 4096, 16384]))
-    plan.fused_step(inv_scale, max_norm)
+    plan.fused_step(inv_scale, max_norm, _lib.RG_STEP_EXPECT_NO_CLIP if one_pass else _lib.RG_STEP_DEFAULT)
     res = plan.result()
     tn = plan.tensor_norms()
     # oracle, tensor by tensor (destination dtypes differ per tensor)
@@ -85,7 +88,12 @@ def test_random_fused_step(seed):
         norms.append(oracle.per_tensor_norms([u])[0])
     assert res.overflow == flag
     if flag:        # a source value did not fit its half type: the step is skipped, nothing is written
-        assert res.skipped == 1 and res.clipped == 0 and all(bool((d == 3.0).all()) for d in dsts)
+        assert res.skipped == 1 and res.clipped == 0
+        if one_pass:
+            for i, (u, d) in enumerate(zip(unscaled, dsts)):
+                assert_bits_equal(d.cpu(), u, f"seed {seed} tensor {i}: unscaled values after an overflow")
+        else:
+            assert all(bool((d == 3.0).all()) for d in dsts)
         return
     total = math.sqrt(sum(n * n for n in norms))
     assert math.isclose(res.norm, total, rel_tol=1e-6, abs_tol=1e-30)
