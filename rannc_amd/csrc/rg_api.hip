@@ -520,7 +520,7 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   if ((flags & RG_STEP_EXPECT_NO_CLIP) && !identity_unless_clipped) {
     // One pass writes the unscaled values while it sums them; only if the decision then says
     // "clip" does a second kernel scale the destination in place.  That kernel's blocks cover
-    // whole chunks, so finding that there is nothing to do costs a few microseconds.
+    // several whole chunks each, so finding that there is nothing to do costs a few microseconds.
     if (all) RG_HIP(hipEventRecord(ev[0], s));
     const int rc1 = tiled_reduce_write(p, a, kModeReduce | kModeWrite, s, max_norm,
                                        (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0, all ? ev[1] : nullptr);
