@@ -211,6 +211,34 @@ class RaNNCModule(_pyrannc.RaNNCModule):
             raise RuntimeError(f"Parameter not found: {name}")       # pyrannc/__init__.py:480-481
         return super().get_param_grad(self.name_to_pid[name], amp_master_param)
 
+    def _sync_orig_params(self, sync_all_ranks=False, sync_grad=False, name_pattern=None):
+        """Write the values the runtime holds back into the user's module (``pyrannc/__init__.py:539-573``): under
+        ZeRO the segments are gathered first; then every named parameter (those whose name contains
+        ``name_pattern``, if given) is overwritten with the root rank's copy, and its gradient too on request."""
+        if not self.ready:
+            return
+        if self.enable_zero:
+            self.sync_param_zero(sync_grad)
+        for name in sorted(self.name_to_param):
+            if name_pattern is not None and name_pattern not in name:
+                continue
+            pid, param = self.name_to_pid[name], self.name_to_param[name]
+            synced = self.sync_param(pid)
+            if synced is not None:
+                with torch.no_grad():
+                    if getattr(param, "distributed", False) and param.size() != synced.size():
+                        param.data = synced          # a placeholder left behind by the sharding: take the full tensor
+                    else:
+                        param.copy_(synced.view(param.size()))
+            if sync_grad:
+                synced_grad = self.sync_param_grad(pid)
+                if synced_grad is not None:
+                    with torch.no_grad():
+                        if param.grad is None:
+                            param.grad = torch.zeros_like(param)
+                        param.grad.copy_(synced_grad.view(param.size()))
+        _pyrannc.barrier()
+
     # ------------------------------------------------------------------ checkpoints
     def state_dict(self, *args, no_hook=False, amp_master_params=True, rank0_only=True, **kwargs):
         r"""

@@ -8,7 +8,7 @@ failures raise ``RuntimeError``.
 """
 from __future__ import annotations
 
-from typing import Dict, Tuple
+from typing import Optional, Dict, Tuple
 
 import torch
 
@@ -231,6 +231,26 @@ class RaNNCModule:
         owner = self._owned_tensor(param_id, amp_master_param)
         grad = owner.grad if owner.grad is not None else torch.zeros_like(owner)
         return self._in_param_shape(grad, param_id)
+
+    def _sync(self, param_id: int, grad: bool) -> Optional[torch.Tensor]:
+        """``ParamStorage::doSyncParam`` + ``bcastParam`` (``src/comp/ParamStorage.cpp:1079-1133``) at one rank: the
+        root's copy of the parameter (or of its gradient, zeros when it has none) as a fresh tensor on the host;
+        ``None`` for a parameter no rank holds (the reference returns an undefined tensor)."""
+        self._check()
+        if param_id not in _param_storage.params:
+            return None
+        param = _param_storage.get_param_tensor(param_id)
+        if grad:
+            src = param.grad if param.grad is not None else torch.zeros_like(param)
+        else:
+            src = param
+        return src.detach().clone().cpu()
+
+    def sync_param(self, param_id: int) -> Optional[torch.Tensor]:
+        return self._sync(param_id, False)
+
+    def sync_param_grad(self, param_id: int) -> Optional[torch.Tensor]:
+        return self._sync(param_id, True)
 
     def undeploy(self) -> None:
         if self._deployed:

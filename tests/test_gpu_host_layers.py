@@ -583,6 +583,37 @@ def test_zero_mode_trains_exactly_like_the_plain_mode(fused, fused_opt):
             assert_bits_equal(b[:a.numel()], a, "zero vs plain")
 
 
+def test_sync_param_and_sync_orig_params():
+    """``sync_param`` / ``sync_param_grad`` (``src/main.cpp:357-366`` -> ``ParamStorage::doSyncParam``) hand back host
+    copies of the parameter and of its gradient (zeros when there is none, ``None`` for an unknown id), and
+    ``_sync_orig_params`` (``pyrannc/__init__.py:539-573``) writes them into the user's module - with one rank: what it
+    already holds, plus a zero gradient for parameters without one."""
+    _pyrannc.clear()
+    torch.manual_seed(31)
+    model = torch.nn.Sequential(torch.nn.Linear(7, 5), torch.nn.Linear(5, 3)).to(DEV)
+    rm = rannc_amd.RaNNCModule(model, None)
+    rm(torch.randn(4, 7, device=DEV)).pow(2).mean().backward()
+    model[1].bias.grad = None
+    before = {n: (p.detach().cpu().clone(), None if p.grad is None else p.grad.detach().cpu().clone().view(p.shape))
+              for n, p in model.named_parameters()}
+    for n, p in model.named_parameters():
+        pid = rm.name_to_pid[n]
+        got = rm.sync_param(pid)
+        assert got.device.type == "cpu" and got.data_ptr() != p.data_ptr()
+        assert_bits_equal(got.view(p.shape), before[n][0], n)
+        gg = rm.sync_param_grad(pid)
+        want = before[n][1] if before[n][1] is not None else torch.zeros_like(before[n][0])
+        assert_bits_equal(gg.view(p.shape), want, n + ".grad")
+    assert rm.sync_param(12345) is None and rm.sync_param_grad(12345) is None
+    rm._sync_orig_params(sync_grad=True, name_pattern="1.")
+    assert model[1].bias.grad is not None and bool((model[1].bias.grad == 0).all())
+    rm._sync_orig_params(sync_grad=True)
+    for n, p in model.named_parameters():
+        assert_bits_equal(p.detach().cpu(), before[n][0], n)
+        want = before[n][1] if before[n][1] is not None else torch.zeros_like(before[n][0])
+        assert_bits_equal(p.grad.detach().cpu().view(p.shape), want, n + ".grad")
+
+
 def test_scale_loss_restores_stashed_gradients_when_the_body_raises():
     torch.manual_seed(5)
     model = torch.nn.Sequential(torch.nn.Linear(8, 8), torch.nn.BatchNorm1d(8)).to(DEV)
