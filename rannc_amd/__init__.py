@@ -137,11 +137,68 @@ class RaNNCModule(_pyrannc.RaNNCModule):
         for t in tensors:
             t.register_hook(on_grad)
 
-    def parameters(self, *args, **kwargs):
-        return self.model.parameters(*args, **kwargs)
+    # ------------------------------------------------------------------ the wrapped module's own interface
+    def _only_used(self, items, from_global: bool, named: bool):
+        """Entries of the wrapped module's parameter / buffer iterators that this process works on
+        (``_param_gen`` / ``_named_param_gen``, ``pyrannc/__init__.py:575-583``); all of them with one rank."""
+        for item in items:
+            tensor = item[1] if named else item
+            if from_global or id(tensor) in self.used_param_ids:
+                yield item
 
-    def named_parameters(self, *args, **kwargs):
-        return self.model.named_parameters(*args, **kwargs)
+    def parameters(self, *args, from_global=False, **kwargs):
+        """Parameters this process holds once deployed (``pyrannc/__init__.py:343-349``)."""
+        if not self.ready:
+            return self.model.parameters(*args, **kwargs)
+        return self._only_used(self.model.parameters(*args, **kwargs), from_global, named=False)
+
+    def named_parameters(self, *args, from_global=False, **kwargs):
+        if not self.ready:
+            return self.model.named_parameters(*args, **kwargs)
+        return self._only_used(self.model.named_parameters(*args, **kwargs), from_global, named=True)
+
+    def buffers(self, *args, **kwargs):
+        """Buffers of the wrapped module (``pyrannc/__init__.py:359-372``).  The reference filters them through the ids
+        of the parameters in use, which no buffer carries, so a deployed module yields none; with one rank the module
+        runs as it is and its buffers are simply its own."""
+        return self.model.buffers(*args, **kwargs)
+
+    def named_buffers(self, *args, **kwargs):
+        return self.model.named_buffers(*args, **kwargs)
+
+    def train(self, mode=True):
+        """A deployed reference module cannot change mode (``pyrannc/__init__.py:323-335``: it only warns); here the
+        wrapped module runs eagerly, so the mode is simply passed on.  Returns ``self`` like ``nn.Module.train``."""
+        self.model.train(mode)
+        return self
+
+    def eval(self):
+        return self.train(False)
+
+    def enable_dropout(self, enable):
+        """Switch dropout layers on or off without touching the rest of the module's mode
+        (``pyrannc/__init__.py:510-521``; the reference flips the flag inside its traced graph)."""
+        for m in self.model.modules():
+            if isinstance(m, torch.nn.modules.dropout._DropoutNd):
+                m.train(bool(enable))
+
+    def to(self, *args, **kwargs):
+        """Ignored with a warning, as in the reference (``pyrannc/__init__.py:312-317``): where the parameters live
+        is the runtime's business.  Move the model before wrapping it."""
+        logger.warning("to() was ignored. A RaNNC model cannot be moved across devices.")
+        return self
+
+    def cuda(self, *args, **kwargs):
+        """Ignored with a warning (``pyrannc/__init__.py:319-324``)."""
+        logger.warning("cuda() was ignored. A RaNNC model cannot be moved across devices.")
+        return self
+
+    def __getattr__(self, attr):
+        """Anything this wrapper does not define is looked up on the wrapped module (``pyrannc/__init__.py:526-537``)."""
+        model = self.__dict__.get("model")
+        if model is None or not hasattr(model, attr):
+            raise AttributeError(f"This model has no attribute '{attr}'")
+        return getattr(model, attr)
 
     # ------------------------------------------------------------------ per-step API
     def _setup_amp_params(self):

@@ -133,3 +133,44 @@ def test_module_requires_amp_for_zero():
     import rannc_amd
     with pytest.raises(ValueError, match="enable_apex_amp"):
         rannc_amd.RaNNCModule(torch.nn.Linear(2, 2), enable_zero=True)
+
+
+def test_module_passes_the_wrapped_models_interface_through():
+    """What ``pyrannc.RaNNCModule`` offers besides the step calls (``pyrannc/__init__.py:312-372, 510-537``): ``to`` /
+    ``cuda`` are ignored, unknown attributes come from the wrapped module, parameter and buffer iterators, ``train`` /
+    ``eval`` / ``enable_dropout`` reach the module.  None of it needs a GPU before the first forward call."""
+    import rannc_amd
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = torch.nn.Linear(3, 2)
+            self.drop = torch.nn.Dropout(0.5)
+            self.register_buffer("steps", torch.zeros(1))
+            self.marker = "hello"
+
+        def forward(self, x):
+            return self.drop(self.lin(x))
+
+        def describe(self, k):
+            return f"net-{k}"
+
+    net = Net()
+    rm = rannc_amd.RaNNCModule(net, None)
+    assert rm.to("cpu") is rm and rm.cuda() is rm                      # ignored, as in the reference
+    assert rm.marker == "hello" and rm.describe(3) == "net-3"
+    with pytest.raises(AttributeError, match="no attribute"):
+        rm.no_such_thing
+    assert [n for n, _ in rm.named_parameters()] == ["lin.weight", "lin.bias"]
+    assert len(list(rm.parameters())) == 2
+    assert [n for n, _ in rm.named_buffers()] == ["steps"] and len(list(rm.buffers())) == 1
+    assert rm.eval() is rm and not net.training and not net.drop.training
+    rm.enable_dropout(True)
+    assert net.drop.training and not net.lin.training                  # only the dropout layers change
+    assert rm.train() is rm and net.training
+    # once deployed the iterators keep to the parameters this process works on (all of them with one rank)
+    rm.ready, rm.used_param_ids = True, {id(net.lin.weight)}
+    assert [n for n, _ in rm.named_parameters()] == ["lin.weight"]
+    assert [n for n, _ in rm.named_parameters(from_global=True)] == ["lin.weight", "lin.bias"]
+    assert len(list(rm.parameters())) == 1
+    rm.ready = False
