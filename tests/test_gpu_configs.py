@@ -189,3 +189,46 @@ def test_c5_zero_flat_buffer_roundtrip(total, nseg):
     torch.cuda.synchronize()
     assert torch.equal(back.view(torch.int16), flat.view(torch.int16)), "round trip is not the identity"
     unflatten.close()
+
+
+def test_single_tensor_beyond_two_to_the_31_elements():
+    """One tensor of 2^31 + 4099 fp16 elements: chunk and tile offsets inside a tensor are 64-bit.  The fused step
+    through a plan and through the allocation-free entry point, and the plan-free cast copy, are checked against
+    torch on the device element for element (the unscale by a power of two is exact, the clip is one fp32 multiply)."""
+    n = 2 ** 31 + 4099
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    x = torch.empty(n, dtype=torch.float16, device=DEV)
+    step = 2 ** 28
+    for lo in range(0, n, step):                         # filled in pieces: no fp32 temporary of the full size
+        hi = min(n, lo + step)
+        x[lo:hi] = (torch.randn(hi - lo, generator=gen, device=DEV) * 1e-3 * 4096.0).to(torch.float16)
+    out = torch.zeros(n, dtype=torch.float32, device=DEV)
+    inv, max_norm = 1.0 / 4096.0, 1.0
+    plan = TensorPlan([x], [out])
+    plan.fused_step(inv, max_norm)
+    res = plan.result()
+    assert res.overflow == 0 and res.clipped == 1
+    sq = 0.0
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        sq += float(((x[lo:hi].float() * inv).double() ** 2).sum())
+    assert math.isclose(res.norm, float(torch.tensor(math.sqrt(sq), dtype=torch.float32)), rel_tol=REL)
+    coef = torch.tensor(res.coef, dtype=torch.float32, device=DEV)
+    inv_t = torch.tensor(inv, dtype=torch.float32, device=DEV)
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        assert bool(torch.equal(out[lo:hi], (x[lo:hi].float() * inv_t) * coef)), f"elements {lo}..{hi}"
+    first = out[-8192:].clone()
+    # the allocation-free entry point: same decision, same bits
+    out.zero_()
+    res_dev = torch.zeros(8, dtype=torch.int32, device=DEV)
+    _lib.fused_step_static(x.data_ptr(), out.data_ptr(), n, _lib.RG_F16, _lib.RG_F32, inv, max_norm, 0, res_dev.data_ptr(), 0,
+                           torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert bool(torch.equal(out[-8192:], first)) and bool(torch.equal(out[:8192], (x[:8192].float() * inv_t) * coef))
+    # plan-free cast copy across the 2^31 boundary
+    _lib.scale_cast_single(x.data_ptr(), out.data_ptr(), n, _lib.RG_F16, _lib.RG_F32, 1.0, 0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for lo in (0, 2 ** 31 - 5000, n - 9000):
+        assert bool(torch.equal(out[lo:lo + 9000], x[lo:lo + 9000].float()))
+    plan.close()
