@@ -327,3 +327,30 @@ def test_direct_step_skips_on_overflow_and_without_clip_call():
     for m, s0 in zip(masters, snap):
         assert torch.equal(m, s0)
     assert amp._amp_state.loss_scalers[0].loss_scale() == 128.0
+
+
+@pytest.mark.gpu
+def test_optimizer_step_on_a_tensor_beyond_two_to_the_31_elements():
+    """Plain SGD on one parameter of 2^31 + 4099 elements: the optimizer kernel's offsets inside a tensor are 64-bit.
+    ``p - lr * g`` evaluated by torch on the device, slice by slice, is the yardstick (2e-6 relative, the bar of the
+    optimizer step)."""
+    dev = torch.device("cuda", 0)
+    n = 2 ** 31 + 4099
+    gen = torch.Generator(device=dev).manual_seed(9)
+    p = torch.nn.Parameter(torch.empty(n, device=dev))
+    g = torch.empty(n, device=dev)
+    step = 2 ** 28
+    with torch.no_grad():
+        for lo in range(0, n, step):
+            hi = min(n, lo + step)
+            p[lo:hi] = torch.randn(hi - lo, generator=gen, device=dev)
+            g[lo:hi] = torch.randn(hi - lo, generator=gen, device=dev)
+    before = p.detach().clone()
+    p.grad = g
+    opt = FusedSGD([p], lr=0.25)
+    opt.step()
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        for lo in range(0, n, step):                     # every element, slice by slice
+            hi = min(n, lo + step)
+            torch.testing.assert_close(p[lo:hi], before[lo:hi] - 0.25 * g[lo:hi], rtol=2e-6, atol=1e-7)
