@@ -160,3 +160,32 @@ def test_random_overflow_positions(seed):
     for s, d, (_, dd) in zip(srcs_cpu, dsts, pairs):
         assert_bits_equal(d.cpu(), oracle.unscale_and_check([s], inv_scale, dd)[0][0], "written on overflow")
     plan.close()
+
+
+@pytest.mark.parametrize("one_pass", [False, True])
+def test_thousands_of_tiny_tensors(one_pass):
+    """3000 tensors of 0 to 40 elements (biases, layer-norm vectors), mixed dtypes, packed into one fp32 bucket at
+    running-sum offsets: nearly every chunk is a ragged sliver and most write tiles are empty."""
+    rng = random.Random(77)
+    g = torch.Generator().manual_seed(77)
+    sizes = [rng.randint(0, 40) for _ in range(3000)]
+    srcs_cpu = [(torch.randn(n, generator=g) * 0.05 * 256.0).to(rng.choice(DTS)) for n in sizes]
+    srcs = _place(srcs_cpu, rng)
+    total = sum(sizes)
+    bucket = torch.full((total + 3,), 5.0, dtype=torch.float32, device=DEV)[3:]
+    dsts, off = [], 0
+    for n in sizes:
+        dsts.append(bucket.narrow(0, off, n))
+        off += n
+    plan = TensorPlan(srcs, dsts)
+    plan.fused_step(1.0 / 256.0, 0.5, _lib.RG_STEP_EXPECT_NO_CLIP if one_pass else _lib.RG_STEP_DEFAULT)
+    res, tn = plan.result(), plan.tensor_norms()
+    want = oracle.fused_step(srcs_cpu, ["f32"] * len(srcs_cpu), 1.0 / 256.0, 0.5)
+    assert res.overflow == want.overflow == 0 and res.clipped == 1
+    assert math.isclose(res.norm, want.norm, rel_tol=1e-6)
+    for a, b in zip(tn, want.tensor_norms):
+        assert math.isclose(a, b, rel_tol=1e-6, abs_tol=1e-30)
+    unscaled = oracle.fused_step(srcs_cpu, ["f32"] * len(srcs_cpu), 1.0 / 256.0, math.inf).buckets["f32"]
+    unscaled.mul_(float(res.coef))
+    assert_bits_equal(bucket.cpu(), unscaled, "bucket of tiny tensors")
+    plan.close()
