@@ -70,7 +70,7 @@ constexpr int kBlockThreads = 256;                               // 4 wavefronts
 // Elements a thread has in flight per loop iteration.  Measured on MI355X: a read-only pass
 // is fastest with deep unrolling over 8-16K-element chunks, a pass that also writes with
 // shallow unrolling over small tiles.
-constexpr int kReduceElemsPerThread = RG_REDUCE_ELEMS_PER_THREAD;
+constexpr int kReduceElemsPerThread = RG_REDUCE_ELEMS_PER_THREAD;   // of fp32; twice as many 16-bit elements (same bytes in flight)
 constexpr int kWriteElemsPerThread = RG_WRITE_ELEMS_PER_THREAD;
 constexpr int kWriteThreads = RG_WRITE_THREADS;                  // block size of write-only passes
 constexpr int kWriteTileElems = RG_WRITE_TILE_ELEMS;             // writing passes cut each chunk into tiles of this size

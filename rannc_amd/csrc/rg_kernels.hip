@@ -49,7 +49,8 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   constexpr bool kReduce = (MODE & kModeReduce) != 0;
   constexpr bool kAcc = (MODE & kModeAccumulate) != 0;   // dst = round_dst(float(dst) + x * scale)
   constexpr int E = (SS == 4 || (kWrite && DS == 4)) ? 4 : 8;   // elements per lane per instruction
-  constexpr int kPerThread = kWrite ? kWriteElemsPerThread : kReduceElemsPerThread;
+  // a read-only pass keeps 128 bytes of source in flight per lane (eight 16-byte loads) whatever the element size
+  constexpr int kPerThread = kWrite ? kWriteElemsPerThread : kReduceElemsPerThread * (4 / SS);
   constexpr int U = kPerThread >= E ? kPerThread / E : 1;      // instructions in flight per lane
   constexpr int AS = kWrite ? DS : SS;
   constexpr unsigned kPeel = kWrite ? kWriteAlignBytes : kAlignBytes;
