@@ -31,7 +31,7 @@ FUSED_OPS = ("fused_step", "fused_step_noclip", "fused_step_noclip_2pass", "over
              "copy_back", "unflatten_back", "grad_norm", "zero")
 C5_OPS = ("c5_unflatten", "c5_master_cast", "c5_copy_back", "c5_repack")
 OPTIM_OPS = ("adam", "sgd", "adam_from_model_grads")
-ALL_OPS = ("all",) + FUSED_OPS + C5_OPS + OPTIM_OPS + ("api_step",)
+ALL_OPS = ("all",) + FUSED_OPS + C5_OPS + OPTIM_OPS + ("api_step", "graph_step")
 
 
 def parse_args():
@@ -627,6 +627,75 @@ def _api_step_leg(args, key: str, scale_numel: float) -> dict:
     return out
 
 
+# ----------------------------------------------------------------------------- optimizer phase decided on the device
+
+def bench_device_decided_phase(args, key: str) -> dict:
+    """Unscale + flag + norm + clip decision (``rg_step_begin`` + ``rg_step_decide``), the device-side Adam step count
+    and the Adam step that reads the scaled bf16 gradients through the gate: nothing is read back by the host, so the
+    phase can also be recorded in a HIP graph.  Reports microseconds per phase for the eager calls and for replays."""
+    import torch
+    from rannc_amd.fused_optim import FusedAdam
+    from rannc_amd.multi_tensor import TensorPlan, stream_handle
+    from rannc_amd.workloads import step_config
+    cfg = step_config(key)
+    dev = torch.device("cuda", 0)
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    shapes = [sh for _, sh in cfg.params]
+    masters = [torch.nn.Parameter(torch.randn(sh, device=dev, generator=gen) * 0.02) for sh in shapes]
+    models = [m.detach().to(torch.bfloat16) for m in masters]
+    grads = [(torch.randn(sh, device=dev, generator=gen) * 1e-2 * 256.0).to(torch.bfloat16) for sh in shapes]
+    n = sum(m.numel() for m in masters)
+    flat = torch.zeros(n, device=dev)                    # master-gradient bucket: part of the plan, never written here
+    views, off = [], 0
+    for m in masters:
+        views.append(flat.narrow(0, off, m.numel()))
+        off += m.numel()
+    plan = TensorPlan(grads, views)
+    opt = FusedAdam(masters, lr=1e-4, capturable=True)
+    opt.set_model_copies(masters, models)
+    opt.set_grad_sources(masters, grads)
+    opt.grad_scale, opt.gate = 1.0 / 256.0, plan.plan.result_device_ptr()
+
+    def phase():
+        s = stream_handle(dev)
+        plan.plan.step_begin(1.0 / 256.0, s)
+        plan.plan.step_decide(1.0, 0, s)
+        opt.step()
+
+    def per_call(fn, k):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(k):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / k * 1e6
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        phase()                                          # allocates the optimizer state: outside any capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    k = max(args.steps, 100)
+    eager = per_call(phase, k)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        phase()
+    replay = per_call(graph.replay, k)
+    res = plan.result()
+    out = {"workload": key, "op": "optimizer_phase_device_decided",
+           "what": "rg_step_begin + rg_step_decide + rg_adam_clock_advance + rg_adam_step_clocked (gated, reads the scaled "
+                   "bf16 gradients, writes the bf16 model copy); no host read-back",
+           "tensors": len(shapes), "elements": n, "eager_us_per_phase": round(eager, 1),
+           "graph_replay_us_per_phase": round(replay, 1), "steps": k, "clipped": bool(res.clipped), "overflow": int(res.overflow)}
+    plan.close()
+    del opt, masters, models, grads, flat, views
+    torch.cuda.empty_cache()
+    return out
+
+
 # ----------------------------------------------------------------------------- main
 
 def headline_line(args, e: dict, w_desc: dict, dtype: str) -> dict:
@@ -699,6 +768,10 @@ def main() -> int:
         print(json.dumps(bench_optimizer(args, args.workload or "c2_bert_large", torch, dev)), flush=True)
         return 0
 
+    if args.op == "graph_step":
+        print(json.dumps(bench_device_decided_phase(args, args.workload or "c1_mlp")), flush=True)
+        return 0
+
     if args.op == "api_step":
         print(json.dumps(bench_api_step(args, args.workload or "c4_resnet152x2")), flush=True)
         return 0
@@ -762,6 +835,8 @@ def main() -> int:
                             "us_per_step": r["value"], "device_us_per_step": r["device_us_per_step"],
                             "host_only_us_per_step": r["host_us_per_step"], "host_us_per_call": r["host_only"]["us_per_call"],
                             "tensors": r["config"]["tensors"], "steps": sub_args.steps})
+        for k3 in ("c1_mlp", "c4_resnet152x2"):
+            configs.append(bench_device_decided_phase(args, k3))
         out["configs"] = configs
 
     if not args.no_cpu_baseline and key != "c5_zero_flat":

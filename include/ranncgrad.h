@@ -294,6 +294,26 @@ typedef struct rg_adam_args {
 } rg_adam_args;
 int rg_adam_step(rg_optim* opt, const rg_adam_args* args, void* stream);
 
+/* The same step with its step count on the device, for callers that record the optimizer phase in a HIP graph
+ * (a count passed by value would be frozen into the graph).  No counterpart in the reference, whose optimizer is
+ * torch.optim's; torch's own graph-capturable Adam keeps `step` on the device in the same way.
+ * An rg_adam_clock is 32 bytes of device memory owned by the caller (one per parameter group), zeroed before
+ * the first step.  rg_adam_clock_advance launches one thread that adds 1 to `step` and stores the two factors
+ * that depend on it, -lr / (1 - beta1^step) and sqrt(1 - beta2^step), computed in double as rg_adam_step
+ * computes them on the host - unless `gate` (optional) says the step was skipped, in which case nothing
+ * changes.  rg_adam_step_clocked is rg_adam_step reading those factors from the clock; args->step is ignored.
+ * Call order on one stream: [rg_fused_step | rg_step_begin ...] -> rg_adam_clock_advance -> rg_adam_step_clocked. */
+typedef struct rg_adam_clock {
+  int64_t step;        /* steps taken so far */
+  float neg_step_size; /* -lr / (1 - beta1^step) */
+  float bias2_sqrt;    /* sqrt(1 - beta2^step) */
+  float step_f32;      /* `step` again as a float (the form torch keeps state["step"] in) */
+  int32_t pad[3];
+} rg_adam_clock;
+int rg_adam_clock_advance(rg_adam_clock* clock_dev, double lr, double beta1, double beta2, const rg_step_result* gate,
+                          int device, void* stream);
+int rg_adam_step_clocked(rg_optim* opt, const rg_adam_args* args, const rg_adam_clock* clock_dev, void* stream);
+
 /* Arithmetic of torch.optim.SGD:
  *   g = grad * grad_scale; g = -g if maximize; g = g + wd * p if wd != 0
  *   momentum != 0:  buf = g on the first step of a buffer (first_step), else

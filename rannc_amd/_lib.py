@@ -79,6 +79,8 @@ SIGNATURES = {
     "rg_optim_update_pointers": (_i, [_vp, _pvp, _pvp, _pvp, _pvp, _pvp, _vp]),
     "rg_optim_destroy": (_i, [_vp]),
     "rg_adam_step": (_i, [_vp, C.POINTER(AdamArgs), _vp]),
+    "rg_adam_step_clocked": (_i, [_vp, C.POINTER(AdamArgs), _vp, _vp]),
+    "rg_adam_clock_advance": (_i, [_vp, C.c_double, C.c_double, C.c_double, _vp, _i, _vp]),
     "rg_sgd_step": (_i, [_vp, C.POINTER(SgdArgs), _vp]),
     "rg_plan_enable_timing": (_i, [_vp, _i]),
     "rg_plan_timing_stride": (_i, [_vp, _i]),
@@ -305,6 +307,15 @@ def _ptr_array(ptrs: Optional[Sequence[Optional[int]]], n: int):
     return (C.c_void_p * max(n, 1))(*[p if p else None for p in ptrs])
 
 
+ADAM_CLOCK_BYTES = 32     # sizeof(rg_adam_clock): int64 step, float neg_step_size, float bias2_sqrt, float step_f32, pad
+
+
+def adam_clock_advance(clock_ptr: int, lr: float, beta1: float, beta2: float, gate: int, device: int, stream: int = 0) -> None:
+    """One thread on the device: the clock's step count + 1 and the factors that depend on it - unless ``gate``
+    (a result block's device address, or 0) says the step was skipped."""
+    check(lib.rg_adam_clock_advance(_vp(clock_ptr), lr, beta1, beta2, _vp(gate or None), device, _vp(stream)))
+
+
 class OptimTable:
     """Owner of one ``rg_optim``: parameter / gradient / state / model-copy pointers of the
     tensors one optimizer launch updates."""
@@ -332,6 +343,14 @@ class OptimTable:
                   stream: int = 0) -> None:
         a = AdamArgs(lr, beta1, beta2, eps, weight_decay, step, int(decoupled), int(maximize), grad_scale, gate or None)
         check(lib.rg_adam_step(self._handle, C.byref(a), _vp(stream)))
+
+    def adam_step_clocked(self, clock_ptr: int, lr: float, beta1: float, beta2: float, eps: float, weight_decay: float,
+                          decoupled: bool = False, maximize: bool = False, grad_scale: float = 1.0, gate: int = 0,
+                          stream: int = 0) -> None:
+        """``adam_step`` with the step count and the factors that depend on it read from an ``rg_adam_clock`` on
+        the device (``adam_clock_advance`` updates it), so that the launch can be replayed from a HIP graph."""
+        a = AdamArgs(lr, beta1, beta2, eps, weight_decay, 0, int(decoupled), int(maximize), grad_scale, gate or None)
+        check(lib.rg_adam_step_clocked(self._handle, C.byref(a), _vp(clock_ptr), _vp(stream)))
 
     def sgd_step(self, lr: float, momentum: float = 0.0, dampening: float = 0.0, weight_decay: float = 0.0,
                  nesterov: bool = False, maximize: bool = False, first_step: bool = False, grad_scale: float = 1.0,

@@ -50,6 +50,7 @@ struct OptConst {
 struct OptArgs {
   const OptChunkRec* chunks;
   const StepResult* gate;
+  const rg_adam_clock* clock;   // Adam only, optional: the step-dependent factors live on the device
   int32_t tile_elems;
   int32_t tiles_per_chunk;
   OptConst c;
@@ -203,6 +204,11 @@ __global__ __launch_bounds__(OptShape<ALGO>::kThreads) void optim_kernel(OptArgs
     if (a.gate->skipped != 0) return;
     coef = a.gate->coef;
   }
+  if (ALGO == kAdam && a.clock != nullptr) {
+    // written by adam_clock_kernel earlier on the same stream
+    a.c.neg_step_size = a.clock->neg_step_size;
+    a.c.bias2_sqrt = a.clock->bias2_sqrt;
+  }
   const unsigned bid = blockIdx.x;
   const OptChunkRec r = a.chunks[bid / (unsigned)a.tiles_per_chunk];
   const int tile = (int)(bid % (unsigned)a.tiles_per_chunk);
@@ -232,6 +238,20 @@ __global__ __launch_bounds__(OptShape<ALGO>::kThreads) void optim_kernel(OptArgs
   RG_OPT(RG_F16, RG_F32)
   RG_OPT(RG_BF16, RG_F32)
 #undef RG_OPT
+}
+
+// One thread: the next step of a device-resident Adam step count and the two factors that depend on it,
+// computed as the host path computes them (in double).  A step the gate says was skipped does not count.
+__global__ void adam_clock_kernel(rg_adam_clock* clock, double lr, double beta1, double beta2, const StepResult* gate) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  if (gate != nullptr && gate->skipped != 0) return;
+  const int64_t step = clock->step + 1;
+  const double bias1 = 1.0 - pow(beta1, (double)step);
+  const double bias2 = 1.0 - pow(beta2, (double)step);
+  clock->step = step;
+  clock->neg_step_size = (float)(-(lr / bias1));
+  clock->bias2_sqrt = (float)sqrt(bias2);
+  clock->step_f32 = (float)step;
 }
 
 }  // namespace
@@ -439,13 +459,14 @@ RG_API int rg_optim_update_pointers(rg_optim* o, void* const* param, const void*
 
 template <int ALGO>
 static int launch_optim(const rg_optim* o, const OptConst& c, const rg_step_result* gate, int64_t bytes_per_elem,
-                        void* stream) {
+                        void* stream, const rg_adam_clock* clock = nullptr) {
   if (o->n_chunks == 0) return RG_OK;
   DeviceGuard guard(o->device);
   OptArgs a;
   memset(&a, 0, sizeof(a));
   a.chunks = o->d_chunks;
   a.gate = reinterpret_cast<const StepResult*>(gate);
+  a.clock = clock;
   a.tile_elems = OptShape<ALGO>::kTileElems;
   a.tiles_per_chunk = (int32_t)((o->chunk_elems + OptShape<ALGO>::kTileElems - 1) / OptShape<ALGO>::kTileElems);
   a.c = c;
@@ -461,24 +482,25 @@ static int launch_optim(const rg_optim* o, const OptConst& c, const rg_step_resu
   return RG_OK;
 }
 
-RG_API int rg_adam_step(rg_optim* o, const rg_adam_args* g, void* stream) {
+static int adam_step(rg_optim* o, const rg_adam_args* g, const rg_adam_clock* clock, void* stream, const char* op) {
   if (o == nullptr || g == nullptr) {
-    set_error("rg_adam_step: null argument");
+    set_error("%s: null argument", op);
     return RG_EINVAL;
   }
   if (!o->has_state1 || !o->has_state2) {
-    set_error("rg_adam_step: the table has no exp_avg / exp_avg_sq pointers");
+    set_error("%s: the table has no exp_avg / exp_avg_sq pointers", op);
     return RG_EINVAL;
   }
-  if (g->step < 1 || !(g->lr >= 0.0) || !(g->eps >= 0.0) || !(g->beta1 >= 0.0 && g->beta1 < 1.0) ||
+  const int64_t step = clock != nullptr ? 1 : g->step;      // with a clock the count lives on the device
+  if (step < 1 || !(g->lr >= 0.0) || !(g->eps >= 0.0) || !(g->beta1 >= 0.0 && g->beta1 < 1.0) ||
       !(g->beta2 >= 0.0 && g->beta2 < 1.0) || !(g->weight_decay >= 0.0)) {
-    set_error("rg_adam_step: bad hyper-parameters (lr %g betas %g %g eps %g wd %g step %lld)", g->lr, g->beta1, g->beta2,
+    set_error("%s: bad hyper-parameters (lr %g betas %g %g eps %g wd %g step %lld)", op, g->lr, g->beta1, g->beta2,
               g->eps, g->weight_decay, (long long)g->step);
     return RG_EINVAL;
   }
   // The scalar factors as torch/optim/adam.py computes them: in double, from Python floats.
-  const double bias1 = 1.0 - pow(g->beta1, (double)g->step);
-  const double bias2 = 1.0 - pow(g->beta2, (double)g->step);
+  const double bias1 = 1.0 - pow(g->beta1, (double)step);
+  const double bias2 = 1.0 - pow(g->beta2, (double)step);
   const double weight = 1.0 - g->beta1;
   OptConst c;
   memset(&c, 0, sizeof(c));
@@ -493,7 +515,36 @@ RG_API int rg_adam_step(rg_optim* o, const rg_adam_args* g, void* stream) {
   c.neg_step_size = (float)(-(g->lr / bias1));
   c.bias2_sqrt = (float)sqrt(bias2);
   c.eps = (float)g->eps;
-  return launch_optim<kAdam>(o, c, g->gate, 30, stream);
+  return launch_optim<kAdam>(o, c, g->gate, 30, stream, clock);
+}
+
+RG_API int rg_adam_step(rg_optim* o, const rg_adam_args* g, void* stream) {
+  return adam_step(o, g, nullptr, stream, "rg_adam_step");
+}
+
+RG_API int rg_adam_step_clocked(rg_optim* o, const rg_adam_args* g, const rg_adam_clock* clock_dev, void* stream) {
+  if (clock_dev == nullptr) {
+    set_error("rg_adam_step_clocked: null clock");
+    return RG_EINVAL;
+  }
+  return adam_step(o, g, clock_dev, stream, "rg_adam_step_clocked");
+}
+
+RG_API int rg_adam_clock_advance(rg_adam_clock* clock_dev, double lr, double beta1, double beta2, const rg_step_result* gate,
+                                 int device, void* stream) {
+  if (clock_dev == nullptr || (reinterpret_cast<uintptr_t>(clock_dev) & 7u) != 0) {
+    set_error("rg_adam_clock_advance: the clock must be an 8-byte aligned device pointer");
+    return RG_EINVAL;
+  }
+  if (!(lr >= 0.0) || !(beta1 >= 0.0 && beta1 < 1.0) || !(beta2 >= 0.0 && beta2 < 1.0)) {
+    set_error("rg_adam_clock_advance: bad hyper-parameters (lr %g betas %g %g)", lr, beta1, beta2);
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(device);
+  hipLaunchKernelGGL(adam_clock_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), clock_dev, lr, beta1, beta2,
+                     reinterpret_cast<const StepResult*>(gate));
+  RG_HIP(hipGetLastError());
+  return RG_OK;
 }
 
 RG_API int rg_sgd_step(rg_optim* o, const rg_sgd_args* g, void* stream) {

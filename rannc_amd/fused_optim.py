@@ -170,10 +170,63 @@ class FusedAdam(_FusedBase):
 
     _decoupled = False
 
-    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, maximize=False):
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, maximize=False,
+                 capturable=False):
+        """``capturable``: as in ``torch.optim.Adam`` - the step count lives on the device (``state["step"]`` is a
+        0-dim float32 GPU tensor), nothing about a step is decided on the host, and ``step()`` may be recorded in
+        a HIP graph and replayed.  Every parameter of a group must then have a gradient at every step, at the same
+        address (graph capture needs that anyway), and the first ``step()`` - which allocates the state - has to
+        run outside a capture."""
         if lr < 0 or eps < 0 or not 0 <= betas[0] < 1 or not 0 <= betas[1] < 1 or weight_decay < 0:
             raise ValueError("invalid Adam hyper-parameters")
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, maximize=maximize))
+        self.capturable = bool(capturable)
+        self._clocks: Dict[int, torch.Tensor] = {}       # group index -> its rg_adam_clock (8 float32 words on the device)
+
+    def load_state_dict(self, state_dict) -> None:
+        super().load_state_dict(state_dict)
+        self._clocks.clear()          # re-seeded from the loaded ``step`` values by the next step
+
+    def _capturable_step(self, gi: int, group) -> None:
+        """One group's step with its count on the device: advance the clock (one thread), then the update kernel."""
+        params = group["params"]
+        if not params:
+            return
+        grads = [self._grad_of(p) for p in params]
+        if any(g is None for g in grads):
+            raise RuntimeError("a capturable optimizer needs a gradient for every parameter at every step")
+        dev = params[0].device
+        clock = self._clocks.get(gi)
+        if clock is None:
+            counts = set()
+            for p, g in zip(params, grads):
+                self._check_param(p, g)
+                st = self.state[p]
+                if len(st) == 0:
+                    st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                    st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                    counts.add(0)
+                else:
+                    counts.add(int(st["step"]))
+            if len(counts) != 1:
+                raise RuntimeError("a capturable optimizer keeps one step count per group; the loaded counts differ")
+            clock = torch.zeros(_lib.ADAM_CLOCK_BYTES // 4, dtype=torch.float32, device=dev)
+            count = counts.pop()
+            if count:
+                clock.view(torch.int64)[0] = count
+                clock[4] = float(count)
+            for p in params:
+                self.state[p]["step"] = clock[4]          # every parameter's count is the group's, on the device
+            self._clocks[gi] = clock
+        ms = [self.state[p]["exp_avg"] for p in params]
+        vs = [self.state[p]["exp_avg_sq"] for p in params]
+        table = self._table((gi, "capturable"), params, grads, ms, vs)
+        b1, b2 = group["betas"]
+        stream = stream_handle(dev)
+        _lib.adam_clock_advance(clock.data_ptr(), group["lr"], b1, b2, self.gate, dev.index, stream)
+        table.adam_step_clocked(clock.data_ptr(), group["lr"], b1, b2, group["eps"], group["weight_decay"],
+                                decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
+                                gate=self.gate, stream=stream)
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -181,6 +234,10 @@ class FusedAdam(_FusedBase):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        if self.capturable:
+            for gi, group in enumerate(self.param_groups):
+                self._capturable_step(gi, group)
+            return loss
         for gi, group in enumerate(self.param_groups):
             steady = self._steady_grads(gi, group)
             if steady is not None:
@@ -235,8 +292,9 @@ class FusedAdamW(FusedAdam):
 
     _decoupled = True
 
-    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, maximize=False):
-        super().__init__(params, lr, betas, eps, weight_decay, maximize)
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, maximize=False,
+                 capturable=False):
+        super().__init__(params, lr, betas, eps, weight_decay, maximize, capturable)
 
 
 class FusedSGD(_FusedBase):

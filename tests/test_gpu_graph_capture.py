@@ -110,3 +110,139 @@ def test_unscale_pack_zero_and_sgd_replay_from_a_graph():
             assert_bits_equal(c.cpu(), p.cpu().to(torch.float16), f"model copy replay {replay}")
             w.copy_(p.cpu())                              # continue from the GPU's trajectory
     table.close()
+
+
+def test_capturable_adam_matches_the_host_counted_step():
+    """``FusedAdam(capturable=True)`` keeps its step count on the device; run eagerly it must walk the same
+    trajectory as the host-counted optimizer (the factors are computed in double on both sides)."""
+    from rannc_amd.fused_optim import FusedAdam
+    g = torch.Generator().manual_seed(12)
+    shapes = [(30001,), (17,), (4096, 3)]
+    init = [torch.randn(s, generator=g) for s in shapes]
+    runs = {}
+    for capturable in (False, True):
+        ps = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+        opt = FusedAdam(ps, lr=1e-2, betas=(0.9, 0.99), weight_decay=0.01, capturable=capturable)
+        gg = torch.Generator().manual_seed(13)
+        for _ in range(5):
+            for p in ps:
+                p.grad = torch.randn(p.shape, generator=gg).to(DEV)
+            opt.step()
+        torch.cuda.synchronize()
+        runs[capturable] = ([p.detach().cpu() for p in ps], [opt.state[p]["exp_avg_sq"].cpu() for p in ps], opt)
+    for a, b in zip(runs[False][0] + runs[False][1], runs[True][0] + runs[True][1]):
+        torch.testing.assert_close(b, a, rtol=2e-6, atol=1e-8)
+    opt = runs[True][2]
+    step = opt.state[opt.param_groups[0]["params"][0]]["step"]
+    assert step.is_cuda and step.dtype == torch.float32 and float(step) == 5.0
+    # the state dict round trip re-seeds the device count
+    ps2 = [torch.nn.Parameter(t.clone()) for t in runs[True][0]]
+    ps2 = [torch.nn.Parameter(p.detach().to(DEV)) for p in ps2]
+    opt2 = FusedAdam(ps2, lr=1e-2, betas=(0.9, 0.99), weight_decay=0.01, capturable=True)
+    import copy
+    opt2.load_state_dict(copy.deepcopy(opt.state_dict()))     # as torch.save / torch.load would hand it over
+    gg = torch.Generator().manual_seed(14)
+    grads = [torch.randn(p.shape, generator=gg).to(DEV) for p in ps2]
+    for p, q, gr in zip(opt.param_groups[0]["params"], ps2, grads):
+        p.grad, q.grad = gr.clone(), gr.clone()
+    opt.step()
+    opt2.step()
+    torch.cuda.synchronize()
+    for p, q in zip(opt.param_groups[0]["params"], ps2):
+        assert_bits_equal(q.detach().cpu(), p.detach().cpu(), "after a state-dict round trip")
+    assert float(opt2.state[ps2[0]]["step"]) == 6.0
+
+
+def test_whole_optimizer_phase_replays_from_a_graph_with_a_skipped_step():
+    """Unscale + flag + norm + clip decision (``rg_step_begin`` / ``rg_step_decide``), the device-side step count and
+    the Adam step that reads the still-scaled fp16 gradients through the gate - one HIP graph, nothing decided on
+    the host.  Replayed with new gradients each time; a replay whose gradients hold an inf must leave the
+    parameters, the moments and the step count as they were; every replay is compared with the CPU oracle."""
+    from oracle import gradpath as oracle
+    from oracle import optim as oracle_optim
+    from rannc_amd.fused_optim import FusedAdam
+    gen = torch.Generator().manual_seed(15)
+    shapes = [(20001,), (5,), (3000, 7)]
+    scale, max_norm = 128.0, 0.5
+    masters_cpu = [torch.randn(s, generator=gen) for s in shapes]
+    m_cpu = [torch.zeros(s) for s in shapes]
+    v_cpu = [torch.zeros(s) for s in shapes]
+    masters = [torch.nn.Parameter(t.clone().to(DEV)) for t in masters_cpu]
+    models = [t.detach().to(torch.float16) for t in masters]
+    static_grads = [torch.zeros(s, dtype=torch.float16, device=DEV) for s in shapes]
+    bucket = [torch.zeros(s, device=DEV) for s in shapes]                 # never written on this route
+    plan = TensorPlan(static_grads, bucket)
+    opt = FusedAdam(masters, lr=1e-2, capturable=True)
+    opt.set_model_copies(masters, models)
+    opt.set_grad_sources(masters, static_grads)
+    opt.grad_scale = 1.0 / scale
+    opt.gate = plan.plan.result_device_ptr()
+
+    def phase():
+        plan.plan.step_begin(1.0 / scale, stream_of())
+        plan.plan.step_decide(max_norm, 0, stream_of())
+        opt.step()
+
+    def stream_of():
+        from rannc_amd.multi_tensor import stream_handle
+        return stream_handle(torch.device(DEV))
+
+    def new_grads(poison=False):
+        out = [(torch.randn(s, generator=gen) * 0.1 * scale).to(torch.float16) for s in shapes]
+        if poison:
+            out[2].view(-1)[1234] = float("inf")
+        return out
+
+    steps_done = 0
+
+    def oracle_step(grads_cpu):
+        nonlocal steps_done
+        want = oracle.fused_step(grads_cpu, ["f32"] * len(shapes), 1.0 / scale, max_norm)
+        if want.overflow:
+            return want
+        steps_done += 1
+        unscaled, _ = oracle.unscale_and_check(grads_cpu, 1.0 / scale)
+        if want.coef is not None:
+            unscaled = [u * torch.tensor(want.coef, dtype=torch.float32) for u in unscaled]
+        oracle_optim.adam_step(masters_cpu, unscaled, m_cpu, v_cpu, steps_done, lr=1e-2)
+        return want
+
+    # one eager step outside the capture: allocates the state and the tables
+    g0 = new_grads()
+    for s, g in zip(static_grads, g0):
+        s.copy_(g)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        phase()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    oracle_step(g0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        phase()
+    # the capture itself does not run the kernels
+    assert float(opt.state[masters[0]]["step"]) == 1.0
+    for replay, poison in enumerate([False, True, False, False]):
+        gc = new_grads(poison)
+        for s, g in zip(static_grads, gc):
+            s.copy_(g)                                         # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle_step(gc)
+        res = plan.result()
+        assert res.overflow == want.overflow == (1 if poison else 0)
+        assert float(opt.state[masters[0]]["step"]) == float(steps_done)
+        for p, w, c in zip(masters, masters_cpu, models):
+            torch.testing.assert_close(p.detach().cpu(), w, rtol=2e-6, atol=2e-8, msg=f"replay {replay}")
+            assert_bits_equal(c.cpu(), p.detach().cpu().to(torch.float16), f"model copy, replay {replay}")
+        for p, w in zip(masters, m_cpu):
+            torch.testing.assert_close(opt.state[p]["exp_avg"].cpu(), w, rtol=2e-6, atol=1e-9)
+        for p, w in zip(masters, masters_cpu):
+            w.copy_(p.detach().cpu())                          # continue from the GPU's trajectory
+        for p, w, x in zip(masters, m_cpu, v_cpu):
+            w.copy_(opt.state[p]["exp_avg"].cpu())
+            x.copy_(opt.state[p]["exp_avg_sq"].cpu())
+    assert steps_done == 4
+    plan.close()
