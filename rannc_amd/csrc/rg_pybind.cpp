@@ -239,6 +239,17 @@ class Optim {
                    reinterpret_cast<const rg_step_result*>(gate)};
     check(rg_adam_step(handle(), &a, current_stream(device_)));
   }
+  // `clock`: a float32 tensor of 8 elements on the device (an rg_adam_clock); advanced, then read by the step
+  void adam_step_clocked(const py::object& clock, double lr, double beta1, double beta2, double eps, double weight_decay,
+                         bool decoupled, bool maximize, float grad_scale, uintptr_t gate) {
+    if (clock.attr("numel")().cast<int64_t>() * clock.attr("element_size")().cast<int64_t>() < (int64_t)sizeof(rg_adam_clock))
+      throw std::invalid_argument("the clock tensor must hold at least 32 bytes");
+    auto* c = reinterpret_cast<rg_adam_clock*>(clock.attr("data_ptr")().cast<uintptr_t>());
+    const auto* g = reinterpret_cast<const rg_step_result*>(gate);
+    check(rg_adam_clock_advance(c, lr, beta1, beta2, g, device_, current_stream(device_)));
+    rg_adam_args a{lr, beta1, beta2, eps, weight_decay, 0, decoupled ? 1 : 0, maximize ? 1 : 0, grad_scale, g};
+    check(rg_adam_step_clocked(handle(), &a, c, current_stream(device_)));
+  }
   void sgd_step(double lr, double momentum, double dampening, double weight_decay, bool nesterov, bool maximize,
                 bool first_step, float grad_scale, uintptr_t gate) {
     rg_sgd_args a{lr, momentum, dampening, weight_decay, nesterov ? 1 : 0, maximize ? 1 : 0, first_step ? 1 : 0, grad_scale,
@@ -451,6 +462,9 @@ PYBIND11_MODULE(_ranncgrad, m) {
            py::arg("model_copies") = py::none())
       .def("adam_step", &Optim::adam_step, py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("eps"),
            py::arg("weight_decay"), py::arg("step"), py::arg("decoupled") = false, py::arg("maximize") = false,
+           py::arg("grad_scale") = 1.0f, py::arg("gate") = (uintptr_t)0)
+      .def("adam_step_clocked", &Optim::adam_step_clocked, py::arg("clock"), py::arg("lr"), py::arg("beta1"), py::arg("beta2"),
+           py::arg("eps"), py::arg("weight_decay"), py::arg("decoupled") = false, py::arg("maximize") = false,
            py::arg("grad_scale") = 1.0f, py::arg("gate") = (uintptr_t)0)
       .def("sgd_step", &Optim::sgd_step, py::arg("lr"), py::arg("momentum") = 0.0, py::arg("dampening") = 0.0,
            py::arg("weight_decay") = 0.0, py::arg("nesterov") = false, py::arg("maximize") = false,

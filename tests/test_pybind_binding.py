@@ -102,6 +102,18 @@ def test_optimizer_table_through_pybind_matches_ctypes():
     assert pl.result()["clipped"] == 1
     oa.sgd_step(0.1, gate=pl.result_device_ptr())
     ob.sgd_step(0.1, gate=pl.result_device_ptr(), stream=stream_handle(dev))
+    # the step with its count on the device: one clock per binding, both continue from step 2
+    clocks = []
+    for _ in range(2):
+        clock = torch.zeros(8, dtype=torch.float32, device=dev)
+        clock.view(torch.int64)[0] = 2
+        clocks.append(clock)
+    oa.adam_step_clocked(clocks[0], 1e-3, 0.9, 0.999, 1e-8, 0.01)
+    _lib.adam_clock_advance(clocks[1].data_ptr(), 1e-3, 0.9, 0.999, 0, 0, stream_handle(dev))
+    ob.adam_step_clocked(clocks[1].data_ptr(), 1e-3, 0.9, 0.999, 1e-8, 0.01, stream=stream_handle(dev))
+    torch.cuda.synchronize()
+    assert int(clocks[0].view(torch.int64)[0]) == 3 and float(clocks[0][4]) == 3.0
+    assert_bits_equal(clocks[0].cpu(), clocks[1].cpu(), "clock")
     for k in "pmvc":
         for x, y in zip(a[k], b[k]):
             assert_bits_equal(x.cpu(), y.cpu(), f"pybind vs ctypes {k}")
