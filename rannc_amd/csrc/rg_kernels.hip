@@ -24,7 +24,7 @@
 #include <type_traits>
 
 // the passes of this file write one stream per launch: see the note on streaming stores in rg_device.h
-#ifndef RG_STREAM_STORE_BITS
+#if !defined(RG_STREAM_STORE_BITS) && !defined(RG_STREAM_STORE_COMPILER_NT)
 #define RG_STREAM_STORE_BITS "sc1 nt"
 #endif
 #include "rg_device.h"
