@@ -28,10 +28,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 HEADLINE = "c3_bert_enlarged"
 
 FUSED_OPS = ("fused_step", "fused_step_noclip", "fused_step_noclip_2pass", "overflow_host_gate", "unscale_pack",
-             "copy_back", "unflatten_back", "grad_norm", "zero")
+             "copy_back", "unflatten_back", "grad_norm", "zero", "accumulate", "unscale_accumulate", "clip_in_place",
+             "consolidate", "zero_staging_pack")
 C5_OPS = ("c5_unflatten", "c5_master_cast", "c5_copy_back", "c5_repack")
 OPTIM_OPS = ("adam", "sgd", "adam_from_model_grads")
-ALL_OPS = ("all",) + FUSED_OPS + C5_OPS + OPTIM_OPS + ("api_step", "graph_step")
+ALL_OPS = ("all",) + FUSED_OPS + C5_OPS + OPTIM_OPS + ("api_step", "graph_step", "ceilings")
 
 
 def parse_args():
@@ -63,6 +64,37 @@ def cpu_model() -> str:
     except OSError:
         pass
     return platform.processor() or "unknown"
+
+
+def gpu_clocks() -> dict:
+    """Clock and power state of GPU 0 as sysfs shows it (the current level of each clock domain is the line
+    marked ``*``), read once before the first kernel so that runs on different boxes can be told apart."""
+    import glob
+    out = {}
+    cards = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_mclk"))
+    if not cards:
+        return {"note": "no sysfs clock files visible"}
+    base = os.path.dirname(cards[0])
+    for name in ("pp_dpm_sclk", "pp_dpm_mclk", "pp_dpm_fclk", "pp_dpm_socclk"):
+        try:
+            lines = [l.strip() for l in open(os.path.join(base, name)) if l.strip()]
+            out[name[len("pp_dpm_"):] + "_levels"] = [l.split(":", 1)[1].strip() for l in lines]
+            cur = [l for l in lines if l.endswith("*")]
+            if cur:
+                out[name[len("pp_dpm_"):]] = cur[0].split(":", 1)[1].replace("*", "").strip()
+        except OSError:
+            pass
+    try:
+        out["perf_level"] = open(os.path.join(base, "power_dpm_force_performance_level")).read().strip()
+    except OSError:
+        pass
+    for hw in glob.glob(os.path.join(base, "hwmon", "hwmon*")):
+        for key, fn in (("power_cap_w", "power1_cap"), ("power_avg_w", "power1_average"), ("power_input_w", "power1_input")):
+            try:
+                out[key] = round(int(open(os.path.join(hw, fn)).read()) / 1e6, 1)
+            except (OSError, ValueError):
+                pass
+    return out
 
 
 # ----------------------------------------------------------------------------- measured traffic
@@ -217,21 +249,21 @@ def run_fused_step(w: StepWorkload, steps: int, warmup: int, op: str = "fused_st
         roof = roofline("pass_kernel<reduce+write, streaming>", (s + d) * n, first_ms * 1e-3,
                         measured_traffic(op, w.key, "pass_kernel<reduce+write>"),
                         note="dominant kernel timed in a second, untimed loop with every stage bracketed",
-                        other_kernels={"combine_tiles+finalize_tensors+finalize_total": {"avg_launch_ms": round(mid_ms, 4)},
+                        other_kernels={"reduce_segments+decide": {"avg_launch_ms": round(mid_ms, 4)},
                                        "pass_kernel<write> gated on the decision (idle)": {"avg_launch_ms": round(last_ms, 4)}})
     else:
-        moved = s * n if (overflow and not clipped and res.skipped) else ((2 * s + d) * n if clipped else (s + d) * n)
         step_bytes = (2 * s + d) * n if clipped else (s + d) * n
         if res.skipped:
-            # the write pass is launched and finds the step skipped: it moves nothing
-            extra["bytes_moved_per_step"] = moved
-            extra["GB/s_on_bytes_moved"] = round(moved / step_s / 1e9, 1)
-            extra["pct_of_hbm_peak_on_bytes_moved"] = round(100.0 * moved / step_s / 1e9 / HBM_PEAK_GBPS, 2)
+            # the write pass is launched and finds the step skipped: the step moves the read pass's bytes only, and
+            # is scored against them
+            step_bytes = s * n
+            extra["note"] = ("skipped on the device: scored against s*N, the bytes the step moves; the write pass's "
+                             "blocks all start, read the decision and exit")
             roof = roofline("pass_kernel<reduce, streaming>", s * n, first_ms * 1e-3,
                             measured_traffic(op, w.key, "pass_kernel<reduce>"),
                             note="the write pass found the step skipped; its idle launch took %.1f us" % (last_ms * 1e3),
                             other_kernels={"pass_kernel<write> (skipped on the device)": {"avg_launch_ms": round(last_ms, 4)},
-                                           "finalize_tensors+finalize_total": {"avg_launch_ms": round(mid_ms, 4)}})
+                                           "reduce_segments+decide": {"avg_launch_ms": round(mid_ms, 4)}})
         else:
             roof = roofline("pass_kernel<write, streaming>", (s + d) * n, last_ms * 1e-3,
                             measured_traffic(op, w.key, "pass_kernel<write>"), launches_timed=len(last_only),
@@ -239,7 +271,7 @@ def run_fused_step(w: StepWorkload, steps: int, warmup: int, op: str = "fused_st
                                 "pass_kernel<reduce>": {"avg_launch_ms": round(first_ms, 4), "algorithmic_bytes_per_launch": s * n,
                                                         "achieved": round(s * n / (first_ms * 1e-3) / 1e9, 1),
                                                         "traffic": measured_traffic(op, w.key, "pass_kernel<reduce>")},
-                                "finalize_tensors+finalize_total": {"avg_launch_ms": round(mid_ms, 4)},
+                                "reduce_segments+decide": {"avg_launch_ms": round(mid_ms, 4)},
                                 "note": "from a second, untimed loop of the same steps with all stages bracketed"})
     return entry(w.key, op, step_s, step_bytes, roof, clipped=clipped, overflow=overflow, skipped=int(res.skipped),
                  norm=res.norm, coef=res.coef, steps=steps, elements_per_s=round(n / step_s, 1), **extra)
@@ -279,6 +311,21 @@ def run_plan_op(w: StepWorkload, op: str, steps: int, warmup: int) -> dict:
         fn, nbytes, kernel = w.plan.grad_norm, s * n, "pass_kernel<reduce>"
     elif op == "zero":
         fn, nbytes, kernel = w.plan.zero, d * n, "pass_kernel<write> (zero fill)"
+    elif op in ("accumulate", "unscale_accumulate"):
+        # dst += src * scale: the destination is read and written; the second form also reports flag and norm
+        w.bucket.zero_()
+        if op == "accumulate":
+            fn, kernel = (lambda: w.plan.accumulate(w.cfg.inv_scale)), "pass_kernel<write+accumulate>"
+        else:
+            fn, kernel = (lambda: w.plan.unscale_accumulate(w.cfg.inv_scale)), "pass_kernel<reduce+write+accumulate>"
+        nbytes = (s + 2 * d) * n
+    elif op == "clip_in_place":
+        # RaNNCModule.clip_grad_norm on gradients that are already unscaled: read pass over the bucket, decision,
+        # in-place multiply
+        plan = TensorPlan(w.views, w.views)
+        cleanup.append(plan)
+        w.plan.scale_cast(w.cfg.inv_scale)
+        fn, nbytes, kernel = (lambda: plan.fused_step(1.0, 1e-30)), 3 * d * n, "pass_kernel<reduce> + pass_kernel<write>"
     elif op == "copy_back":
         # fp32 masters (the packed bucket holds fp32 values after a step) -> model parameters in the gradient dtype
         mdt = w.grads[0].dtype if w.grads[0].dtype != torch.float32 else torch.bfloat16
@@ -303,9 +350,78 @@ def run_plan_op(w: StepWorkload, op: str, steps: int, warmup: int) -> dict:
     for p in cleanup:
         p.close()
     extra = {}
-    if op == "unscale_pack":
-        extra["note"] = "launch time = pass + combine_tiles + finalize kernels (whole operation, device events)"
+    if op in ("unscale_pack", "unscale_accumulate"):
+        extra["note"] = "launch time = pass + reduce_segments + decide kernels (whole operation, device events)"
+    if op == "clip_in_place":
+        extra["note"] = ("every step clips (max_norm 1e-30: the values shrink towards zero, the traffic is the same): "
+                         "read d, then read d + write d")
     return entry(w.key, op, wall, nbytes, roofline(kernel, nbytes, dev_s, measured_traffic(op, w.key, kernel), **extra), steps=steps)
+
+
+def run_host_layer_op(w: StepWorkload, op: str, steps: int, warmup: int) -> dict:
+    """Two per-step operations of the registry, driven through the mirror of the reference's classes on parameters
+    shaped like the workload: ``consolidate`` = ``GradConsolidation::consolidate`` (``src/comp/ParamStorage.cpp:118-179``:
+    every gradient copied into its bucket view), ``zero_staging_pack`` = ``allReduceParamGradsZero`` at one rank
+    (``:440-520``: gradients packed into zero-padded staging buffers, fp16/bf16 widened to fp32, and copied back)."""
+    import torch
+    from rannc_amd.param_storage import GradConsolidation, ParamStorage
+    n, s = w.n, w.s
+    params = [torch.nn.Parameter(torch.empty(g.shape, dtype=g.dtype, device=w.dev)) for g in w.grads]
+    st = ParamStorage()
+    ids = {}
+    for i, p in enumerate(params):
+        st.register_param(id(p), p)
+        ids[f"p{i:05d}"] = id(p)
+    if op == "consolidate":
+        con = GradConsolidation(st, [id(p) for p in params], False, False)
+
+        def fn():
+            for p, g in zip(params, w.grads):      # backward left fresh gradients outside the buckets
+                p.grad = g
+            con.consolidate()
+        nbytes, kernel = 2 * s * n, "pass_kernel<write> (raw copy)"
+    else:
+        st.deploy("g", ids, enable_zero=True, allreduce_amp_master_params=True)
+        for p, g in zip(params, w.grads):
+            p.grad = g
+        wide = 4 if w.grads[0].dtype == torch.float16 else s       # the reference widens fp16 only (ParamStorage.cpp:483-486)
+
+        def fn():
+            st.allreduce_param_grads_zero("g")
+        nbytes, kernel = 2 * (s + wide) * n, "pass_kernel<write> x2 (pack into staging, copy back)"
+    wall, dev_s = timed(fn, steps, warmup, 10)
+    if op != "consolidate":
+        st.undeploy("g")
+    return entry(w.key, op, wall, nbytes, roofline(kernel, nbytes, dev_s, None,
+                 note="launch time = all launches of the operation (device events); ms_per_step is wall time including "
+                      "the host's per-parameter bookkeeping"), steps=steps, tensors=len(params))
+
+
+# ----------------------------------------------------------------------------- yardsticks
+
+def run_ceilings(steps: int, warmup: int, nbytes: int = 1 << 30) -> list:
+    """The library's yardstick kernels (``rg_ceiling_kernel``): the passes' access patterns over flat 1 GiB arrays."""
+    import torch
+    from rannc_amd import _lib
+    from rannc_amd.multi_tensor import stream_handle
+    dev = torch.device("cuda", 0)
+    arrays = [torch.empty(nbytes // 4, dtype=torch.float32, device=dev).fill_(1.0) for _ in range(4)]
+    ptrs = [a.data_ptr() for a in arrays]
+    out = []
+    for name, kind, moved in (("read", 0, 1.0), ("fill", 1, 1.0), ("copy_f32", 2, 2.0), ("copy_f32_nt", 5, 2.0),
+                              ("widen_bf16_f32", 3, 1.5), ("adam_streams", 4, 7.0)):
+        def fn():
+            _lib.ceiling_kernel(kind, ptrs, nbytes, 0, stream_handle(dev))
+        wall, dev_s = timed(fn, steps, warmup, 20)
+        b = int(moved * nbytes)
+        out.append({"workload": "flat_1GiB", "op": "ceiling_" + name, "ms_per_step": round(dev_s * 1e3, 4),
+                    "algorithmic_bytes_per_step": b, "GB/s": round(b / dev_s / 1e9, 1),
+                    "pct_of_hbm_peak": round(100.0 * b / dev_s / 1e9 / HBM_PEAK_GBPS, 2), "steps": steps})
+        if name == "adam_streams":
+            arrays[0].fill_(1.0)
+    del arrays
+    torch.cuda.empty_cache()
+    return out
 
 
 # ----------------------------------------------------------------------------- ZeRO flat buffer (config 5)
@@ -728,9 +844,11 @@ def run_one(args, key: str, op: str, steps: int, warmup: int) -> tuple:
         e = run_fused_step(w, steps, warmup, op)
     elif op == "overflow_host_gate":
         e = run_overflow_host_gate(w, steps, warmup)
+    elif op in ("consolidate", "zero_staging_pack"):
+        e = run_host_layer_op(w, op, steps, warmup)
     else:
         e = run_plan_op(w, op, steps, warmup)
-    if op not in ("copy_back", "unflatten_back"):
+    if op not in ("copy_back", "unflatten_back", "consolidate", "zero_staging_pack"):
         e.setdefault("tuned_write_order", w.write_order)
     desc = w.describe()
     dtype = f"{w.cfg.grad_dtype}->{w.cfg.bucket_dtype} (fp32 arithmetic)"
@@ -772,14 +890,21 @@ def main() -> int:
         print(json.dumps(bench_device_decided_phase(args, args.workload or "c1_mlp")), flush=True)
         return 0
 
+    if args.op == "ceilings":
+        print(json.dumps({"metric": "achieved HBM GB/s of the yardstick kernels", "unit": "GB/s", "clocks": gpu_clocks(),
+                          "configs": run_ceilings(max(args.steps, 20), args.warmup)}), flush=True)
+        return 0
+
     if args.op == "api_step":
         print(json.dumps(bench_api_step(args, args.workload or "c4_resnet152x2")), flush=True)
         return 0
 
+    clocks = gpu_clocks()
     key = args.workload or HEADLINE
     op = args.op if args.op not in (None, "all") else ("c5_unflatten" if key == "c5_zero_flat" else "fused_step")
     e, desc, dtype = run_one(args, key, op, args.steps, args.warmup)
     out = headline_line(args, e, desc, dtype)
+    out["clocks"] = clocks
 
     if everything:
         # every other configuration and operation of the path, each measured like the headline (their own step
@@ -790,9 +915,16 @@ def main() -> int:
             ("c3_bert_enlarged", "fused_step_noclip", args.steps), ("c3_bert_enlarged", "unscale_pack", args.steps),
             ("c2_bert_large", "fused_step", sub), ("c2_bert_large", "fused_step_noclip", sub),
             ("c2_bert_large", "fused_step_noclip_2pass", sub), ("c2_bert_large", "unscale_pack", sub),
-            ("c2_bert_large", "copy_back", sub),
+            ("c2_bert_large", "copy_back", sub), ("c2_bert_large", "zero", sub), ("c2_bert_large", "grad_norm", sub),
+            ("c2_bert_large", "accumulate", sub), ("c2_bert_large", "unscale_accumulate", sub),
+            ("c2_bert_large", "clip_in_place", sub), ("c2_bert_large", "consolidate", sub),
+            ("c2_bert_large", "zero_staging_pack", sub),
             ("c4_resnet152x2", "fused_step", sub), ("c4_resnet152x2", "fused_step_noclip", sub),
-            ("c1_mlp", "fused_step", 4 * sub), ("c1_mlp", "unflatten_back", 4 * sub),
+            ("c4_resnet152x2", "unscale_pack", sub), ("c4_resnet152x2", "zero", sub), ("c4_resnet152x2", "grad_norm", sub),
+            ("c4_resnet152x2", "accumulate", sub), ("c4_resnet152x2", "unscale_accumulate", sub),
+            ("c4_resnet152x2", "clip_in_place", sub), ("c4_resnet152x2", "consolidate", sub),
+            ("c4_resnet152x2", "zero_staging_pack", sub),
+            ("c1_mlp", "fused_step", 4 * sub), ("c1_mlp", "fused_step_noclip", 4 * sub), ("c1_mlp", "unflatten_back", 4 * sub),
         ]
         configs = []
         cur_key, w = None, None
@@ -805,9 +937,11 @@ def main() -> int:
                 configs.append(run_fused_step(w, st, args.warmup, op2))
             elif op2 == "overflow_host_gate":
                 configs.append(run_overflow_host_gate(w, st, args.warmup))
+            elif op2 in ("consolidate", "zero_staging_pack"):
+                configs.append(run_host_layer_op(w, op2, st, args.warmup))
             else:
                 configs.append(run_plan_op(w, op2, st, args.warmup))
-            if op2 not in ("copy_back", "unflatten_back"):      # those run on a plan of their own, not tuned
+            if op2 not in ("copy_back", "unflatten_back", "consolidate", "zero_staging_pack"):      # those run on plans of their own, not tuned
                 configs[-1].setdefault("tuned_write_order", w.write_order)
         if w is not None:
             w.close()
@@ -837,6 +971,7 @@ def main() -> int:
                             "tensors": r["config"]["tensors"], "steps": sub_args.steps})
         for k3 in ("c1_mlp", "c4_resnet152x2"):
             configs.append(bench_device_decided_phase(args, k3))
+        configs.extend(run_ceilings(sub, args.warmup))
         out["configs"] = configs
 
     if not args.no_cpu_baseline and key != "c5_zero_flat":

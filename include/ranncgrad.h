@@ -130,6 +130,9 @@ int rg_plan_set_streaming(rg_plan* plan, int mode);
  * contiguous eighth per XCD). */
 int rg_plan_tune(rg_plan* plan, void* stream);
 int rg_plan_write_order(const rg_plan* plan);
+/* Set that order directly (same encoding; RG_EINVAL outside [-1, 65536]): for a caller that has measured it on an
+ * earlier plan of the same layout and must not have this plan's destinations overwritten by another measurement. */
+int rg_plan_set_write_order(rg_plan* plan, int order);
 
 /* ---------------------------------------------------------------- per-step operations */
 
@@ -234,14 +237,17 @@ int rg_read_tensor_norms(rg_plan* plan, float* out_host, void* stream);
  * anything.  It has no counterpart in the reference; it is for callers that cannot call
  * hipMalloc or rg_plan_create: code under HIP graph capture, tight serving loops, harnesses
  * that forbid allocation.  The working memory a plan would own (result block, per-chunk
- * partial sums) is a fixed array of about 3 MiB in the library's device image, one copy per
- * GPU, held until the process ends; numel above RG_STATIC_MAX_NUMEL is rejected with
- * RG_EINVAL.  The kernels overwrite every slot they later read, so nothing needs clearing
- * between calls; calls that overlap on one GPU (two streams, two threads) race on that array
- * and must be serialised by the caller.  Same arithmetic, same launch shapes and therefore
- * the same bits as rg_fused_step on a one-tensor plan; `result_dev` (device memory of the
- * caller, 8-byte aligned, may be NULL) receives the rg_step_result on the stream. */
-#define RG_STATIC_MAX_NUMEL 4294967296LL /* 2^32 elements */
+ * partial sums) is a fixed array of about 4 MiB in the library's device image, one copy per
+ * GPU, held until the process ends.  Limit: RG_STATIC_MAX_SRC_BYTES of source, i.e. 2^32
+ * elements of fp16 / bf16 or 2^31 of fp32 (a chunk is 32 KiB of source whatever the type);
+ * more is rejected with RG_EINVAL.  The kernels overwrite every slot they later read, so
+ * nothing needs clearing between calls; calls that overlap on one GPU (two streams, two
+ * threads) race on that array and must be serialised by the caller.  Same arithmetic, same
+ * chunking and launch shapes and therefore the same bits as rg_fused_step on a one-tensor
+ * plan; `result_dev` (device memory of the caller, 8-byte aligned, may be NULL) receives the
+ * rg_step_result on the stream. */
+#define RG_STATIC_MAX_SRC_BYTES 8589934592LL /* 2^33 */
+#define RG_STATIC_MAX_NUMEL 4294967296LL     /* 2^32 elements of a 16-bit source type */
 int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t numel, int src_dtype, int dst_dtype,
                          float inv_scale, float max_norm, int flags, rg_step_result* result_dev, int device,
                          void* stream);
@@ -346,6 +352,18 @@ int rg_sgd_step(rg_optim* opt, const rg_sgd_args* args, void* stream);
 int rg_plan_enable_timing(rg_plan* plan, int slots);
 int rg_plan_timing_stride(rg_plan* plan, int stride);
 int rg_plan_read_timing(rg_plan* plan, int slot, float ms[4]);
+
+/* Yardstick kernels (no counterpart in the reference): the access patterns of the passes above over flat arrays -
+ * no work table, no tensor boundaries, no sums - with the library's own load / store helpers and launch shapes, so
+ * that a pass can be compared with what its pattern reaches on the same GPU in the same run.  One launch on `stream`.
+ * `nbytes` (a multiple of 16) is the size of the widest stream; every array must be 16-byte aligned.
+ *   kind 0  read only             arrays: src[nbytes], sink[>= 4 bytes, never written in practice]
+ *   kind 1  fill (write only)     arrays: dst[nbytes]
+ *   kind 2  fp32 copy * 1.5       arrays: src[nbytes], dst[nbytes]
+ *   kind 3  bf16 -> fp32 * 0.5    arrays: src[nbytes / 2], dst[nbytes]
+ *   kind 4  Adam's streams        arrays: p, g, m, v [nbytes each]; p, m, v rewritten in place
+ *   kind 5  kind 2 with the compiler's plain nontemporal stores instead of the write passes' cache policy */
+int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, int64_t nbytes, int device, void* stream);
 
 #ifdef __cplusplus
 }

@@ -285,6 +285,8 @@ class RaNNCModule(_pyrannc.RaNNCModule):
                 with torch.no_grad():
                     if getattr(param, "distributed", False) and param.size() != synced.size():
                         param.data = synced          # a placeholder left behind by the sharding: take the full tensor
+                        if hasattr(self.optimizer, "invalidate_tables"):
+                            self.optimizer.invalidate_tables()
                     else:
                         param.copy_(synced.view(param.size()))
             if sync_grad:

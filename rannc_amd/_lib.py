@@ -57,6 +57,7 @@ SIGNATURES = {
     "rg_plan_set_streaming": (_i, [_vp, _i]),
     "rg_plan_tune": (_i, [_vp, _vp]),
     "rg_plan_write_order": (_i, [_vp]),
+    "rg_plan_set_write_order": (_i, [_vp, _i]),
     "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
     "rg_step_begin": (_i, [_vp, _f, _vp]),
     "rg_step_finish": (_i, [_vp, _f, _i, _vp]),
@@ -85,6 +86,7 @@ SIGNATURES = {
     "rg_plan_enable_timing": (_i, [_vp, _i]),
     "rg_plan_timing_stride": (_i, [_vp, _i]),
     "rg_plan_read_timing": (_i, [_vp, _i, C.POINTER(C.c_float)]),
+    "rg_ceiling_kernel": (_i, [_i, _pvp, _i, _i64, _i, _vp]),
 }
 
 
@@ -178,6 +180,9 @@ class Plan:
             lib.rg_plan_destroy(self._handle)
             self._handle = _vp()
 
+    def is_open(self) -> bool:
+        return bool(getattr(self, "_handle", None) is not None and self._handle.value)
+
     def __del__(self):
         try:
             self.close()
@@ -205,6 +210,14 @@ class Plan:
         destinations, waits for the stream).  Returns the order chosen."""
         check(lib.rg_plan_tune(self._handle, _vp(stream)))
         return int(lib.rg_plan_write_order(self._handle))
+
+    @property
+    def write_order(self) -> int:
+        """Order in which the writing passes hand tiles to the XCDs (0 round robin, n runs of n, -1 eighths)."""
+        return int(lib.rg_plan_write_order(self._handle))
+
+    def set_write_order(self, order: int) -> None:
+        check(lib.rg_plan_set_write_order(self._handle, order))
 
     def update_pointers(self, src_ptrs: Optional[Sequence[Optional[int]]],
                         dst_ptrs: Optional[Sequence[Optional[int]]], stream: int = 0) -> None:
@@ -291,6 +304,15 @@ def fused_step_static(src_ptr: int, dst_ptr: int, numel: int, src_dtype: int, ds
     """The fused step over one tensor pair with no plan and no allocation (``rg_fused_step_static``)."""
     check(lib.rg_fused_step_static(_vp(src_ptr or None), _vp(dst_ptr or None), numel, src_dtype, dst_dtype, inv_scale,
                                    max_norm, flags, _vp(result_ptr or None), device, _vp(stream)))
+
+
+CEILING_KINDS = {"read": 0, "fill": 1, "copy_f32": 2, "widen_bf16_f32": 3, "adam_streams": 4, "copy_f32_nt": 5}
+
+
+def ceiling_kernel(kind: int, array_ptrs: Sequence[int], nbytes: int, device: int, stream: int = 0) -> None:
+    """One launch of a yardstick kernel (``rg_ceiling_kernel``) over caller-owned device arrays."""
+    n = len(array_ptrs)
+    check(lib.rg_ceiling_kernel(kind, (_vp * max(n, 1))(*array_ptrs), n, nbytes, device, _vp(stream)))
 
 
 def fill_zero(ptr: int, nbytes: int, device: int, stream: int = 0) -> None:

@@ -116,16 +116,18 @@ class LossScaler:
         if stash.unscale_cache is None:
             from ..param_storage import _PlanCache
             stash.unscale_cache = _PlanCache()
+        if stash.clip_decided:
+            # what the last step decided picks this step's strategy; it is read from the table that took the
+            # decision, before the cache may replace that table by a new one
+            if stash.unscale_plan is not None and stash.unscale_plan.is_open():
+                stash.expect_clip = bool(stash.unscale_plan.result().clipped)
+            stash.clip_decided = False
         # a new table is tuned on the spot, unless the master gradients hold values that are about to be added to
         if all_params:
             stash.unscale_plan = stash.unscale_cache.get_same_shapes("all", model_grads, master_grads, tune_new=not accumulate)
         else:
             stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads, tune_new=not accumulate)
         inv = 1.0 / self._loss_scale
-        if stash.clip_decided:
-            # what the last step decided (still in the table's result block) picks this step's strategy
-            stash.expect_clip = bool(stash.unscale_plan.result().clipped)
-            stash.clip_decided = False
         stash.sums_cover_all = False
         with torch.no_grad():
             if accumulate:
@@ -467,6 +469,15 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
 def zip_params(optimizer):
     """(fp32 master, half model parameter) pairs in stash order (``pyrannc/amp/__init__.py:9-11``); creates the
     masters first if no ``scale_loss`` has run yet."""
+    stash = optimizer._amp_stash
+    pairs = _master_model_pairs(optimizer)
+    if stash.pending_finish:
+        finish_unscale(optimizer)         # callers read master.grad through these pairs
+    return pairs
+
+
+def _master_model_pairs(optimizer):
+    """The pairs themselves, for code that only wants to know which master belongs to which parameter."""
     _lazy_init_maybe_master_weights(optimizer)
     stash = optimizer._amp_stash
     return zip(stash.all_fp32_from_fp16_params, stash.all_fp16_params)
@@ -477,7 +488,7 @@ def register_amp_params(optimizer):
     Under ZeRO the optimizer holds local segments; they are registered under the id of the parameter they are
     a segment of."""
     segment_owner = getattr(optimizer, "param_zero_segment_to_id", {})
-    for master, model_param in zip_params(optimizer):
+    for master, model_param in _master_model_pairs(optimizer):
         owner = segment_owner[model_param] if model_param in segment_owner else id(model_param)
         _pyrannc.register_amp_master_param(owner, master)
 
@@ -486,7 +497,9 @@ def named_master_params(model, optimizer, zero=False):
     """``(name, tensor the optimizer steps on)`` for every parameter (``pyrannc/amp/__init__.py:21-41``): the
     fp32 master of a half parameter, the parameter itself when it already is fp32.  With ``zero`` the tensors
     are local segments and the names come from the module's ``name_to_pid``; otherwise the order is that of
-    ``model.named_parameters()``."""
+    ``model.named_parameters()``.  The reference's tests read the unscaled gradients through it
+    (``p.grad for n, p in named_master_params(...)``, ``test/common.py:86``), so a deferred write of the master
+    gradients is completed first (inside ``zip_params``)."""
     if not hasattr(optimizer._amp_stash, "all_fp32_from_fp16_params"):
         return
     stepped_for = {model_param: master for master, model_param in zip_params(optimizer)}

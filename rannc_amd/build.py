@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_NAME = "libranncgrad.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["rg_kernels.hip", "rg_api.hip", "rg_optim.hip"]
+SOURCES = ["rg_kernels.hip", "rg_api.hip", "rg_optim.hip", "rg_ceilings.hip"]
 
 # -ffp-contract=off: the unscale and clip multiplies must stay two roundings.
 # The packed-fp32 feature is switched off for every HIP translation unit of this project.

@@ -40,7 +40,6 @@ struct rg_plan {
   int xcd_reduce = 64;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
   int xcd_write = 0;                 //   ... when every source sits on the line grid of its destination
   int xcd_write_offgrid = 256;       //   ... when some source does not (see fill_chunk_records)
-  int64_t reduce_tile_factor = 0;    // tile of a reducing + writing pass, in write tiles (0 = per operation)
   float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
   bool sums_describe_dst = false;   // the per-tensor sums on the device are those of the destinations as last written
   std::vector<TensorDesc> host_tensors;
@@ -53,14 +52,13 @@ struct rg_plan {
   char* dev_base = nullptr;
   size_t dev_bytes = 0;
   ChunkRec* d_chunks = nullptr;
-  int64_t* d_tensor_chunk_begin = nullptr;
-  double* d_chunk_sumsq = nullptr;
-  int32_t* d_chunk_bad = nullptr;
-  WavePartial* d_wave_partials = nullptr;   // [n_chunks * max_tiles * wavefronts per tile]: a tiled reduce+write pass
+  Partial* d_partials = nullptr;            // [n_chunks * max tiles per chunk * wavefronts per tile]: what the reducing passes leave
+  int64_t* d_seg_chunk_begin = nullptr;     // [n_segments + 1]
+  int32_t* d_tensor_seg_begin = nullptr;    // [n_tensors + 1]
+  Partial* d_seg_sums = nullptr;            // [n_segments]
   float* d_tensor_norm = nullptr;
-  double* d_tensor_sq = nullptr;
-  int32_t* d_tensor_bad = nullptr;
   StepResult* d_result = nullptr;
+  int n_segments = 0;
 
   // pinned host memory: two chunk-table staging buffers (pointer updates stay stream
   // ordered without a host wait in the common case) and a read-back area
@@ -244,19 +242,6 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   // The Infinity Cache holds 256 MiB: below that a second pass can still hit in cache.
   p->streaming = bytes > (int64_t)256 << 20;
   p->chunk_elems = chunk_elems > 0 ? chunk_elems : default_chunk_elems(total, widest_src);
-  // Tuning knobs of experiment builds, read once per plan (defaults are what measured best on MI355X):
-  //   RG_WRITE_TILE_ELEMS    elements per block of a writing pass (>= 256)
-  //   RG_XCD_REDUCE / _WRITE block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run);
-  //                          unset, writing passes use 0, or runs of 256 when a source is off its destination's line grid
-  //   RG_REDUCE_TILE_FACTOR  tile of a reducing + writing pass, in write tiles (0 = per operation)
-#ifdef RG_TUNING_ENV   // experiment builds only: the shipped library takes no launch shape from the environment
-  if (const char* env = getenv("RG_WRITE_TILE_ELEMS")) p->write_tile_elems = atoll(env);
-  if (const char* env = getenv("RG_XCD_REDUCE")) p->xcd_reduce = atoi(env);
-  if (const char* env = getenv("RG_XCD_WRITE")) p->xcd_write = p->xcd_write_offgrid = atoi(env);
-  if (const char* env = getenv("RG_REDUCE_TILE_FACTOR")) p->reduce_tile_factor = atoll(env);
-#endif
-  if (p->reduce_tile_factor < 0) p->reduce_tile_factor = 0;
-
   p->chunk_begin.assign((size_t)n + 1, 0);
   for (int i = 0; i < n; ++i)
     p->chunk_begin[(size_t)i + 1] = p->chunk_begin[(size_t)i] + (numel[i] + p->chunk_elems - 1) / p->chunk_elems;
@@ -267,6 +252,19 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
     return RG_EINVAL;
   }
 
+  // Segments: the units the partial sums of a tensor are added in (see rg_internal.h).  They depend on the chunk
+  // counts only, so they are laid out once.
+  std::vector<int64_t> seg_chunk_begin;
+  std::vector<int32_t> tensor_seg_begin((size_t)n + 1, 0);
+  for (int i = 0; i < n; ++i) {
+    const int64_t first = p->chunk_begin[(size_t)i], count = p->chunk_begin[(size_t)i + 1] - first;
+    const int64_t per = std::max<int64_t>(kSegmentChunks, (count + kMaxSegmentsPerTensor - 1) / kMaxSegmentsPerTensor);
+    for (int64_t c = 0; c < count; c += per) seg_chunk_begin.push_back(first + c);
+    tensor_seg_begin[(size_t)i + 1] = (int32_t)seg_chunk_begin.size();
+  }
+  p->n_segments = (int)seg_chunk_begin.size();
+  seg_chunk_begin.push_back(p->n_chunks);
+
   // carve one device allocation
   size_t off = 0;
   auto carve = [&off](size_t nbytes) {
@@ -275,18 +273,16 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
     return at;
   };
   const size_t nt = (size_t)(n > 0 ? n : 1), nc = (size_t)(p->n_chunks > 0 ? p->n_chunks : 1);
+  const size_t ns = (size_t)(p->n_segments > 0 ? p->n_segments : 1);
   const size_t o_chunks = carve(nc * sizeof(ChunkRec));
-  const size_t o_begin = carve((nt + 1) * sizeof(int64_t));
-  // a tiled reduce+write pass leaves one partial per tile
+  // a pass that sums while it writes leaves one partial per wavefront of every tile
   if (p->write_tile_elems < kMinWriteTileElems) p->write_tile_elems = kMinWriteTileElems;
   const size_t max_tiles = (size_t)((p->chunk_elems + p->write_tile_elems - 1) / p->write_tile_elems);
-  const size_t o_sumsq = carve(nc * sizeof(double));
-  const size_t o_bad = carve(nc * sizeof(int32_t));
-  const size_t tile_partials = nc * max_tiles * (size_t)(kWriteThreads / 64);   // one per wavefront of every tile
-  const size_t o_wave_partials = carve(tile_partials * sizeof(WavePartial));
+  const size_t o_partials = carve(nc * max_tiles * (size_t)kWaveSlotsPerTile * sizeof(Partial));
+  const size_t o_seg_begin = carve((ns + 1) * sizeof(int64_t));
+  const size_t o_tensor_seg = carve((nt + 1) * sizeof(int32_t));
+  const size_t o_seg_sums = carve(ns * sizeof(Partial));
   const size_t o_tnorm = carve(nt * sizeof(float));
-  const size_t o_tsq = carve(nt * sizeof(double));
-  const size_t o_tbad = carve(nt * sizeof(int32_t));
   const size_t o_result = carve(sizeof(StepResult));
   p->dev_bytes = off;
 
@@ -298,13 +294,11 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   }
   char* b = p->dev_base;
   p->d_chunks = reinterpret_cast<ChunkRec*>(b + o_chunks);
-  p->d_tensor_chunk_begin = reinterpret_cast<int64_t*>(b + o_begin);
-  p->d_chunk_sumsq = reinterpret_cast<double*>(b + o_sumsq);
-  p->d_chunk_bad = reinterpret_cast<int32_t*>(b + o_bad);
-  p->d_wave_partials = reinterpret_cast<WavePartial*>(b + o_wave_partials);
+  p->d_partials = reinterpret_cast<Partial*>(b + o_partials);
+  p->d_seg_chunk_begin = reinterpret_cast<int64_t*>(b + o_seg_begin);
+  p->d_tensor_seg_begin = reinterpret_cast<int32_t*>(b + o_tensor_seg);
+  p->d_seg_sums = reinterpret_cast<Partial*>(b + o_seg_sums);
   p->d_tensor_norm = reinterpret_cast<float*>(b + o_tnorm);
-  p->d_tensor_sq = reinterpret_cast<double*>(b + o_tsq);
-  p->d_tensor_bad = reinterpret_cast<int32_t*>(b + o_tbad);
   p->d_result = reinterpret_cast<StepResult*>(b + o_result);
 
   const size_t stage_bytes = (nc * sizeof(ChunkRec) + 255) / 256 * 256;
@@ -325,7 +319,10 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   if (ok && p->n_chunks > 0)
     ok = hipMemcpy(p->d_chunks, p->stage[0], (size_t)p->n_chunks * sizeof(ChunkRec), hipMemcpyHostToDevice) == hipSuccess;
   if (ok)
-    ok = hipMemcpy(p->d_tensor_chunk_begin, p->chunk_begin.data(), p->chunk_begin.size() * sizeof(int64_t),
+    ok = hipMemcpy(p->d_seg_chunk_begin, seg_chunk_begin.data(), seg_chunk_begin.size() * sizeof(int64_t),
+                   hipMemcpyHostToDevice) == hipSuccess;
+  if (ok)
+    ok = hipMemcpy(p->d_tensor_seg_begin, tensor_seg_begin.data(), tensor_seg_begin.size() * sizeof(int32_t),
                    hipMemcpyHostToDevice) == hipSuccess;
   for (int k = 0; ok && k < 2; ++k) ok = hipEventCreateWithFlags(&p->stage_done[k], hipEventDisableTiming) == hipSuccess;
   if (!ok) {
@@ -401,8 +398,7 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   PassArgs a;
   memset(&a, 0, sizeof(a));
   a.chunks = p->d_chunks;
-  a.chunk_sumsq = p->d_chunk_sumsq;
-  a.chunk_bad = p->d_chunk_bad;
+  a.partials = p->d_partials;
   a.result = nullptr;
   a.n_chunks = p->n_chunks;
   a.tile_elems = (int32_t)p->chunk_elems;
@@ -416,21 +412,21 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   return a;
 }
 
-static FinalizeArgs finalize_args(const rg_plan* p, float max_norm, int ignore_overflow) {
-  FinalizeArgs f;
-  memset(&f, 0, sizeof(f));
-  f.tensor_chunk_begin = p->d_tensor_chunk_begin;
-  f.chunk_sumsq = p->d_chunk_sumsq;
-  f.chunk_bad = p->d_chunk_bad;
-  f.tensor_norm = p->d_tensor_norm;
-  f.tensor_sq = p->d_tensor_sq;
-  f.tensor_bad = p->d_tensor_bad;
-  f.result = p->d_result;
-  f.n_tensors = p->n_tensors;
-  f.max_norm = max_norm;
-  f.ignore_overflow = ignore_overflow;
-  f.partials_per_chunk = 1;
-  return f;
+static ReduceArgs reduce_args(const rg_plan* p, float max_norm, int ignore_overflow, int partials_per_chunk = 1) {
+  ReduceArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partials = p->d_partials;
+  r.seg_chunk_begin = p->d_seg_chunk_begin;
+  r.tensor_seg_begin = p->d_tensor_seg_begin;
+  r.seg_sums = p->d_seg_sums;
+  r.tensor_norm = p->d_tensor_norm;
+  r.result = p->d_result;
+  r.n_tensors = p->n_tensors;
+  r.n_segments = p->n_segments;
+  r.partials_per_chunk = partials_per_chunk;
+  r.max_norm = max_norm;
+  r.ignore_overflow = ignore_overflow;
+  return r;
 }
 
 // Write-only passes cut every chunk into tiles so that more, smaller blocks are in flight.
@@ -457,28 +453,14 @@ static hipError_t launch_scale_if_clipped(const rg_plan* p, hipStream_t s) {
 }
 
 // One pass that both reduces and writes, over tiles of each chunk: every wavefront of every
-// tile leaves its own partial sum; a small kernel folds them into per-chunk sums, which the
-// per-tensor finalize then adds as it does after a read-only pass.
+// tile leaves its own partial sum; two small launches (one for small plans) turn them into the
+// per-tensor norms and the decision.
 static int tiled_reduce_write(rg_plan* p, PassArgs& a, int mode, hipStream_t s, float max_norm = 0.0f,
                               int ignore_overflow = 0, hipEvent_t after_pass = nullptr) {
   split_for_write(p, a);
-  // measured on MI355X: the plain write tile is best now that no block-wide combine ends a tile
-  const int64_t factor = p->reduce_tile_factor > 0 ? p->reduce_tile_factor : 1;
-  if (a.tiles_per_chunk > 1 && factor > 1 && a.tile_elems * factor <= p->chunk_elems) {
-    a.tile_elems = (int32_t)(a.tile_elems * factor);
-    a.tiles_per_chunk = (int32_t)((p->chunk_elems + a.tile_elems - 1) / a.tile_elems);
-  }
-  a.wave_partials = p->d_wave_partials;
   RG_HIP(launch_pass(mode, a, p->streaming, s));
   if (after_pass) RG_HIP(hipEventRecord(after_pass, s));
-  CombineArgs c;
-  c.partials = p->d_wave_partials;
-  c.chunk_sumsq = p->d_chunk_sumsq;
-  c.chunk_bad = p->d_chunk_bad;
-  c.n_chunks = p->n_chunks;
-  c.partials_per_chunk = a.tiles_per_chunk * (kWriteThreads / 64);
-  RG_HIP(launch_combine_tiles(c, s));
-  RG_HIP(launch_finalize(finalize_args(p, max_norm, ignore_overflow), s));
+  RG_HIP(launch_reduce(reduce_args(p, max_norm, ignore_overflow, a.tiles_per_chunk * kWaveSlotsPerTile), p->n_chunks, s));
   return RG_OK;
 }
 
@@ -540,7 +522,7 @@ RG_API int rg_fused_step(rg_plan* p, float inv_scale, float max_norm, int flags,
   a.xcd_run = p->xcd_reduce;
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
   if (all) RG_HIP(hipEventRecord(ev[1], s));
-  RG_HIP(launch_finalize(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
+  RG_HIP(launch_reduce(reduce_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), p->n_chunks, s));
   if (ev) RG_HIP(hipEventRecord(ev[2], s));
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
@@ -571,7 +553,7 @@ RG_API int rg_step_begin(rg_plan* p, float inv_scale, void* stream) {
   PassArgs a = pass_args(p, inv_scale);
   a.xcd_run = p->xcd_reduce;
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
-  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 0), s));
+  RG_HIP(launch_reduce(reduce_args(p, 0.0f, 0), p->n_chunks, s));
   p->begun_inv_scale = inv_scale;
   return RG_OK;
 }
@@ -585,7 +567,7 @@ RG_API int rg_step_finish(rg_plan* p, float max_norm, int flags, void* stream) {
   }
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  RG_HIP(launch_finalize_total(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
+  RG_HIP(launch_decide(reduce_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
   PassArgs a = pass_args(p, p->begun_inv_scale);
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
@@ -603,8 +585,8 @@ RG_API int rg_step_decide(rg_plan* p, float max_norm, int flags, void* stream) {
     return RG_EINVAL;
   }
   DeviceGuard guard(p->device);
-  RG_HIP(launch_finalize_total(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0),
-                               reinterpret_cast<hipStream_t>(stream)));
+  RG_HIP(launch_decide(reduce_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0),
+                       reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;   // the begin stays pending: rg_step_finish may still write the gradients
 }
 
@@ -632,7 +614,7 @@ RG_API int rg_step_apply_clip(rg_plan* p, float max_norm, int flags, void* strea
   }
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  RG_HIP(launch_finalize_total(finalize_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
+  RG_HIP(launch_decide(reduce_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
   RG_HIP(launch_scale_if_clipped(p, s));
   p->sums_describe_dst = false;                          // the destinations are about to change
   return RG_OK;
@@ -687,7 +669,7 @@ RG_API int rg_grad_norm(rg_plan* p, void* stream) {
   a.norm_of_source = 1;
   a.xcd_run = p->xcd_reduce;
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
-  RG_HIP(launch_finalize(finalize_args(p, 0.0f, 1), s));
+  RG_HIP(launch_reduce(reduce_args(p, 0.0f, 1), p->n_chunks, s));
   return RG_OK;
 }
 
@@ -759,6 +741,15 @@ RG_API int rg_plan_write_order(const rg_plan* p) {
   return p == nullptr ? 0 : (p->offgrid ? p->xcd_write_offgrid : p->xcd_write);
 }
 
+RG_API int rg_plan_set_write_order(rg_plan* p, int order) {
+  if (p == nullptr || order < -1 || order > 65536) {
+    set_error("rg_plan_set_write_order: bad arguments (order %d)", order);
+    return RG_EINVAL;
+  }
+  p->xcd_write = p->xcd_write_offgrid = order;
+  return RG_OK;
+}
+
 RG_API int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t numel, int src_dtype, int dst_dtype,
                                 float scale, int device, void* stream) {
   const int ss = elem_size(src_dtype), ds = elem_size(dst_dtype);
@@ -808,15 +799,15 @@ RG_API int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t nume
 // ---------------------------------------------------------------------------- allocation-free fused step
 
 // Working memory of rg_fused_step_static: what a plan keeps in its own allocation (result
-// block, per-tensor norm, one partial sum and flag per chunk), for one tensor pair of at most
-// RG_STATIC_MAX_NUMEL elements.  Every GPU the library runs on holds its own copy of this
+// block, per-tensor norm, segment sums, one partial per chunk), for one tensor pair of at most
+// RG_STATIC_MAX_SRC_BYTES of source.  Every GPU the library runs on holds its own copy of this
 // array until the process ends; host code only ever uses the per-device address looked up below.
-constexpr int64_t kStaticMaxChunks = RG_STATIC_MAX_NUMEL / RG_DEFAULT_CHUNK_ELEMS;
+constexpr int64_t kStaticMaxChunks = RG_STATIC_MAX_SRC_BYTES / (2 * RG_DEFAULT_CHUNK_ELEMS);   // 32 KiB of source per chunk
 constexpr size_t kStaticResultOff = 0;        // StepResult
-constexpr size_t kStaticTensorOff = 256;      // float norm @0, double sq @8, int32 bad @16
-constexpr size_t kStaticSumsqOff = 512;       // double[kStaticMaxChunks]
-constexpr size_t kStaticBadOff = kStaticSumsqOff + (size_t)kStaticMaxChunks * sizeof(double);
-constexpr size_t kStaticScratchBytes = kStaticBadOff + (size_t)kStaticMaxChunks * sizeof(int32_t);
+constexpr size_t kStaticTensorOff = 256;      // float norm
+constexpr size_t kStaticSegOff = 512;         // Partial[kMaxSegmentsPerTensor]
+constexpr size_t kStaticPartialsOff = kStaticSegOff + (size_t)kMaxSegmentsPerTensor * sizeof(Partial);
+constexpr size_t kStaticScratchBytes = kStaticPartialsOff + (size_t)kStaticMaxChunks * sizeof(Partial);
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
@@ -847,9 +838,9 @@ RG_API int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t nume
     set_error("rg_fused_step_static: bad arguments (dtypes %d->%d, numel %lld)", src_dtype, dst_dtype, (long long)numel);
     return RG_EINVAL;
   }
-  if (numel > (int64_t)RG_STATIC_MAX_NUMEL) {
-    set_error("rg_fused_step_static: %lld elements exceed the limit of %lld; use a plan (rg_fused_step)",
-              (long long)numel, (long long)RG_STATIC_MAX_NUMEL);
+  if (numel > (int64_t)RG_STATIC_MAX_SRC_BYTES / ss) {
+    set_error("rg_fused_step_static: %lld elements of %d bytes exceed the limit of %lld source bytes; use a plan (rg_fused_step)",
+              (long long)numel, ss, (long long)RG_STATIC_MAX_SRC_BYTES);
     return RG_EINVAL;
   }
   if (!(inv_scale == inv_scale) || inv_scale == 0.0f) {
@@ -871,8 +862,12 @@ RG_API int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t nume
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 
   // the launch shapes of a one-tensor plan, so that both give the same bits
-  const int64_t chunk = default_chunk_elems(numel);
+  const int64_t chunk = default_chunk_elems(numel, ss);
   const int64_t n_chunks = (numel + chunk - 1) / chunk;
+  if (n_chunks > kStaticMaxChunks) {      // cannot happen below the size limit; the array's bound is checked all the same
+    set_error("rg_fused_step_static: %lld chunks exceed the working memory", (long long)n_chunks);
+    return RG_EINVAL;
+  }
   const bool streaming = numel * (ss + ds) > ((int64_t)256 << 20);
   const int64_t head = numel > 0 ? tensor_head(src_dev, dst_dev, ss, ds) : 0;
   const bool offgrid = numel > head &&
@@ -888,8 +883,7 @@ RG_API int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t nume
   a.single_chunk_elems = chunk;
   a.single_head = head;
   a.peel_heads = head != 0 ? 1 : 0;
-  a.chunk_sumsq = reinterpret_cast<double*>(base + kStaticSumsqOff);
-  a.chunk_bad = reinterpret_cast<int32_t*>(base + kStaticBadOff);
+  a.partials = reinterpret_cast<Partial*>(base + kStaticPartialsOff);
   a.n_chunks = n_chunks;
   a.tile_elems = (int32_t)chunk;
   a.tiles_per_chunk = 1;
@@ -897,21 +891,21 @@ RG_API int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t nume
   a.xcd_run = 64;
   RG_HIP(launch_pass(kModeReduce, a, streaming, s));
 
-  FinalizeArgs f;
+  ReduceArgs f;
   memset(&f, 0, sizeof(f));
+  f.partials = a.partials;
   f.single_chunks = n_chunks;
-  f.chunk_sumsq = a.chunk_sumsq;
-  f.chunk_bad = a.chunk_bad;
+  f.single_seg_chunks = std::max<int64_t>(kSegmentChunks, (n_chunks + kMaxSegmentsPerTensor - 1) / kMaxSegmentsPerTensor);
+  f.n_segments = (int)((n_chunks + f.single_seg_chunks - 1) / f.single_seg_chunks);
+  f.seg_sums = reinterpret_cast<Partial*>(base + kStaticSegOff);
   f.tensor_norm = reinterpret_cast<float*>(base + kStaticTensorOff);
-  f.tensor_sq = reinterpret_cast<double*>(base + kStaticTensorOff + 8);
-  f.tensor_bad = reinterpret_cast<int32_t*>(base + kStaticTensorOff + 16);
   f.result = reinterpret_cast<StepResult*>(base + kStaticResultOff);
   f.result_copy = result_dev;
   f.n_tensors = 1;
+  f.partials_per_chunk = 1;
   f.max_norm = max_norm;
   f.ignore_overflow = (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0;
-  f.partials_per_chunk = 1;
-  RG_HIP(launch_finalize(f, s));
+  RG_HIP(launch_reduce(f, n_chunks, s));
 
   a.result = f.result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;

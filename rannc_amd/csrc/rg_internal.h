@@ -98,12 +98,25 @@ constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial st
 // Pass selection for the chunk kernel.
 enum : int { kModeReduce = 1, kModeWrite = 2, kModeAccumulate = 4 };  // accumulate: dst = round(dst + x * scale)
 
-// What one wavefront of a pass that reduces and writes leaves behind: one 16-byte store.
-struct alignas(16) WavePartial {
+// A partial sum of squares with the inf/NaN flag of the elements it covers: what a block of the read-only pass
+// and every wavefront of a pass that sums while it writes leave behind, in one 16-byte store.
+struct alignas(16) Partial {
   double sumsq;
   int32_t bad;
   int32_t pad;
 };
+constexpr int kWaveSlotsPerTile = kWriteThreads / 64;   // partials one tile of a pass that sums while it writes leaves
+
+// From partials to the decision in two launches.  The partials of a tensor are cut into segments of whole chunks
+// (kSegmentChunks each; more for a tensor that would otherwise have over kMaxSegmentsPerTensor of them): one block
+// per segment adds its partials in a fixed order, then a single block adds each tensor's segment sums (one thread
+// per tensor), rounds to n_t = float(sqrt(sum)), adds double(n_t)^2 over the tensors and takes the clip decision.
+// Plans with few segments and partials run both stages in that single block: one launch.
+constexpr int64_t kSegmentChunks = 256;
+constexpr int kMaxSegmentsPerTensor = 64;
+constexpr int kDecideThreads = 1024;
+constexpr int kSmallReduceSegments = 64;        // the one-launch form: at most this many segments ...
+constexpr int64_t kSmallReducePartials = 16384; // ... and this many partials
 
 struct PassArgs {
   const ChunkRec* chunks;        // [n_chunks]; null = one tensor described by `single`
@@ -113,9 +126,7 @@ struct PassArgs {
   int64_t single_head;           // elements before the first aligned chunk boundary
   int32_t xcd_run;               // block -> XCD mapping, see pass_kernel
   int32_t peel_heads;            // writing passes: some destination starts off a boundary
-  double* chunk_sumsq;           // [n_chunks] written by a read-only reducing pass
-  int32_t* chunk_bad;            // [n_chunks]
-  WavePartial* wave_partials;    // [blocks * wavefronts per block] written by a pass that reduces and writes
+  Partial* partials;             // read-only pass: [n_chunks]; pass that sums while it writes: one per wavefront of every tile
   const StepResult* result;      // non-null: take coef / overflow gate from the device
   int64_t n_chunks;
   int32_t tile_elems;            // elements one block handles (== chunk_elems unless the pass splits chunks)
@@ -129,37 +140,31 @@ struct PassArgs {
   int32_t chunks_per_block;      // launch_gated_pass only: consecutive chunks one block walks through
 };
 
-struct FinalizeArgs {
-  const int64_t* tensor_chunk_begin;  // [n_tensors + 1]; null = one tensor made of `single_chunks` chunks
+struct ReduceArgs {
+  const Partial* partials;            // chunk-major: chunk c owns [c * partials_per_chunk, (c + 1) * partials_per_chunk)
+  const int64_t* seg_chunk_begin;     // [n_segments + 1]; null = one tensor cut into segments of single_seg_chunks chunks
+  const int32_t* tensor_seg_begin;    // [n_tensors + 1]; null = one tensor that owns every segment
   int64_t single_chunks;
-  const double* chunk_sumsq;
-  const int32_t* chunk_bad;
+  int64_t single_seg_chunks;
+  Partial* seg_sums;                  // [n_segments]
   float* tensor_norm;                 // [n_tensors]
-  double* tensor_sq;                  // [n_tensors]
-  int32_t* tensor_bad;                // [n_tensors]
   StepResult* result;
   rg_step_result* result_copy;        // optional second place the decision is written to (caller's memory)
   int32_t n_tensors;
+  int32_t n_segments;
+  int32_t partials_per_chunk;         // 1 after the read-only pass, else tiles per chunk * kWaveSlotsPerTile
   float max_norm;
-  int32_t ignore_overflow;  // overflow is reported but neither gates the clip nor the write
-  int32_t partials_per_chunk;  // 1, or the tiles per chunk of a tiled reducing pass
-};
-
-struct CombineArgs {
-  const WavePartial* partials;   // [n_chunks * partials_per_chunk], chunk-major
-  double* chunk_sumsq;        // [n_chunks]
-  int32_t* chunk_bad;
-  int64_t n_chunks;
-  int32_t partials_per_chunk;
+  int32_t ignore_overflow;            // overflow is reported but neither gates the clip nor the write
 };
 
 // streaming: nontemporal loads/stores (data far larger than the caches).
 hipError_t launch_pass(int mode, const PassArgs& a, bool streaming, hipStream_t stream);
 // A whole-chunk write pass that runs only if result->clipped is set, launched with few blocks.
 hipError_t launch_gated_pass(const PassArgs& a, bool streaming, hipStream_t stream);
-hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream);
-hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream);
-hipError_t launch_combine_tiles(const CombineArgs& a, hipStream_t stream);
+// partials -> segment sums -> per-tensor norms -> decision (n_chunks: chunks the partials cover)
+hipError_t launch_reduce(const ReduceArgs& a, int64_t n_chunks, hipStream_t stream);
+// segment sums (left by an earlier launch_reduce) -> per-tensor norms -> decision for a.max_norm
+hipError_t launch_decide(const ReduceArgs& a, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
 
 void set_error(const char* fmt, ...);

@@ -239,15 +239,10 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
   // A pass that reduces and writes leaves one partial per wavefront (no block-wide combine at
   // the end of a tile that only lives a few microseconds); a read-only pass one per block.
   constexpr bool kWavePartials = (MODE & kModeReduce) != 0 && (MODE & kModeWrite) != 0;
-  constexpr int kSlots = kWavePartials ? T / 64 : 1;
+  constexpr int kSlots = kWavePartials ? kWaveSlotsPerTile : 1;
   if (start >= end) {
-    if constexpr (kWavePartials) {
-      if (threadIdx.x < kSlots) a.wave_partials[slot_id * kSlots + threadIdx.x] = WavePartial{0.0, 0, 0};
-    } else if (MODE & kModeReduce) {
-      if (threadIdx.x == 0) {
-        a.chunk_sumsq[slot_id] = 0.0;
-        a.chunk_bad[slot_id] = 0;
-      }
+    if constexpr ((MODE & kModeReduce) != 0) {
+      if (threadIdx.x < kSlots) a.partials[slot_id * kSlots + threadIdx.x] = Partial{0.0, 0, 0};
     }
     return;
   }
@@ -330,7 +325,7 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
         bad = __any(mine) ? 1 : 0;
       }
       // sum and flag leave in one 16-byte store
-      if ((threadIdx.x & 63) == 0) a.wave_partials[slot_id * kSlots + (threadIdx.x >> 6)] = WavePartial{s, bad, 0};
+      if ((threadIdx.x & 63) == 0) a.partials[slot_id * kSlots + (threadIdx.x >> 6)] = Partial{s, bad, 0};
     } else {
       // One partial per block, the wavefronts combined through LDS in index order.
       __shared__ double wave_sum[kWaves];
@@ -349,10 +344,7 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
         }
         bad = __syncthreads_or(mine);
       }
-      if (threadIdx.x == 0) {
-        a.chunk_sumsq[slot_id] = total;
-        a.chunk_bad[slot_id] = bad;
-      }
+      if (threadIdx.x == 0) a.partials[slot_id] = Partial{total, bad, 0};
     }
   }
 }
@@ -400,8 +392,9 @@ __global__ __launch_bounds__(PassThreads<kModeWrite>::value) void gated_pass_ker
   for (int64_t c = first; c < last; ++c) pass_block<kModeWrite, NT, PEEL>(a, (unsigned)c, coef);
 }
 
-// Fixed-order sum of one value per thread over the block: DPP row scans inside each
-// wavefront, then the wavefront totals through LDS in index order.
+// Fixed-order sum of one value per thread over a block of W wavefronts: DPP row scans inside each
+// wavefront, then the wavefront totals through LDS in index order.  Every thread returns the total.
+template <int W>
 __device__ __forceinline__ void block_sum_or(double& s, int& bad, double* lds_sum, int* lds_bad) {
   s = wave_total(s);
   bad = __any(bad) ? 1 : 0;
@@ -410,110 +403,148 @@ __device__ __forceinline__ void block_sum_or(double& s, int& bad, double* lds_su
     lds_bad[threadIdx.x >> 6] = bad;
   }
   __syncthreads();
-  s = (lds_sum[0] + lds_sum[1]) + (lds_sum[2] + lds_sum[3]);
-  bad = lds_bad[0] | lds_bad[1] | lds_bad[2] | lds_bad[3];
+  double total = 0.0;
+  int any = 0;
+#pragma unroll
+  for (int w = 0; w < W; w += 4) {
+    total += (lds_sum[w] + lds_sum[w + 1]) + (lds_sum[w + 2] + lds_sum[w + 3]);
+    any |= lds_bad[w] | lds_bad[w + 1] | lds_bad[w + 2] | lds_bad[w + 3];
+  }
+  s = total;
+  bad = any;
   __syncthreads();
 }
 
-// After a pass that left one partial per wavefront of every tile: wavefront w of the grid adds
-// the partials of chunk w in a fixed order into the chunk's slot of the per-chunk arrays, so
-// that the per-tensor kernel below sees the same number of values whatever pass produced them
-// (a large tensor has tens of thousands of tile partials, too many for its one block).
-__global__ __launch_bounds__(kBlockThreads) void combine_tiles_kernel(CombineArgs a) {
-  const int64_t c = (int64_t)blockIdx.x * (kBlockThreads / 64) + (threadIdx.x >> 6);
-  if (c >= a.n_chunks) return;
-  const int lane = threadIdx.x & 63;
-  const WavePartial* ps = a.partials + c * a.partials_per_chunk;
-  double s = 0.0;
-  int bad = 0;
-  for (int i = lane; i < a.partials_per_chunk; i += 64) {
-    const WavePartial w = ps[i];
-    s += w.sumsq;
-    bad |= w.bad;
-  }
-  s = wave_total(s);
-  bad = __any(bad) ? 1 : 0;
-  if (lane == 0) {
-    a.chunk_sumsq[c] = s;
-    a.chunk_bad[c] = bad;
+// Chunks [c0, c1) of segment `seg`.
+__device__ __forceinline__ void segment_chunks(const ReduceArgs& a, int seg, int64_t& c0, int64_t& c1) {
+  if (a.seg_chunk_begin != nullptr) {
+    c0 = a.seg_chunk_begin[seg];
+    c1 = a.seg_chunk_begin[seg + 1];
+  } else {
+    c0 = (int64_t)seg * a.single_seg_chunks;
+    c1 = c0 + a.single_seg_chunks;
+    if (c1 > a.single_chunks) c1 = a.single_chunks;
   }
 }
 
-// Block t reduces tensor t's chunk sums (thread-strided with four independent loads in
-// flight, then a fixed tree) to n_t = float(sqrt(sum)).
-__global__ __launch_bounds__(kBlockThreads) void finalize_tensors_kernel(FinalizeArgs a) {
-  __shared__ double lds_sum[kBlockThreads / 64];
-  __shared__ int lds_bad[kBlockThreads / 64];
-  const int t = blockIdx.x;
+// Stage 1: block b adds the partials of segment b (thread-strided with four independent loads in
+// flight, then a fixed tree).
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void reduce_segments_kernel(ReduceArgs a) {
+  __shared__ double lds_sum[THREADS / 64];
+  __shared__ int lds_bad[THREADS / 64];
+  int64_t c0, c1;
+  segment_chunks(a, (int)blockIdx.x, c0, c1);
+  const int64_t end = c1 * a.partials_per_chunk;
+  int64_t i = c0 * a.partials_per_chunk + threadIdx.x;
   double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
   int bad = 0;
-  // partials_per_chunk > 1: the pass left one partial per tile, laid out chunk-major
-  const int64_t first = a.tensor_chunk_begin ? a.tensor_chunk_begin[t] : 0;
-  const int64_t end = (a.tensor_chunk_begin ? a.tensor_chunk_begin[t + 1] : a.single_chunks) * a.partials_per_chunk;
-  int64_t c = first * a.partials_per_chunk + threadIdx.x;
-  for (; c + 3 * kBlockThreads < end; c += 4 * kBlockThreads) {
-    const double v0 = a.chunk_sumsq[c], v1 = a.chunk_sumsq[c + kBlockThreads];
-    const double v2 = a.chunk_sumsq[c + 2 * kBlockThreads], v3 = a.chunk_sumsq[c + 3 * kBlockThreads];
-    const int b0 = a.chunk_bad[c], b1 = a.chunk_bad[c + kBlockThreads];
-    const int b2 = a.chunk_bad[c + 2 * kBlockThreads], b3 = a.chunk_bad[c + 3 * kBlockThreads];
-    s0 += v0; s1 += v1; s2 += v2; s3 += v3;
-    bad |= b0 | b1 | b2 | b3;
+  for (; i + 3 * THREADS < end; i += 4 * THREADS) {
+    const Partial w0 = a.partials[i], w1 = a.partials[i + THREADS];
+    const Partial w2 = a.partials[i + 2 * THREADS], w3 = a.partials[i + 3 * THREADS];
+    s0 += w0.sumsq; s1 += w1.sumsq; s2 += w2.sumsq; s3 += w3.sumsq;
+    bad |= w0.bad | w1.bad | w2.bad | w3.bad;
   }
-  for (; c < end; c += kBlockThreads) {
-    s0 += a.chunk_sumsq[c];
-    bad |= a.chunk_bad[c];
+  for (; i < end; i += THREADS) {
+    const Partial w = a.partials[i];
+    s0 += w.sumsq;
+    bad |= w.bad;
   }
   double s = (s0 + s1) + (s2 + s3);
-  block_sum_or(s, bad, lds_sum, lds_bad);
-  if (threadIdx.x == 0) {
-    const float n = (float)sqrt(s);
-    a.tensor_norm[t] = n;
-    a.tensor_sq[t] = (double)n * (double)n;
-    a.tensor_bad[t] = bad;
-  }
+  block_sum_or<THREADS / 64>(s, bad, lds_sum, lds_bad);
+  if (threadIdx.x == 0) a.seg_sums[blockIdx.x] = Partial{s, bad, 0};
 }
 
-// One block adds double(n_t)^2 over all tensors in a fixed order and derives the clip
-// decision.  It runs as its own launch after finalize_tensors_kernel: a kernel boundary
-// is a far cheaper device-wide barrier here than per-block fences, whose L2 write-back
-// across the eight XCDs cost about 30 us for a few hundred blocks.
-__global__ __launch_bounds__(kBlockThreads) void finalize_total_kernel(FinalizeArgs a) {
-  __shared__ double lds_sum[kBlockThreads / 64];
-  __shared__ int lds_bad[kBlockThreads / 64];
-  double s0 = 0.0, s1 = 0.0;
+// Stage 2, one block: thread t adds the segment sums of tensor t in order (eight loads in flight) and rounds
+// to n_t = float(sqrt(sum)), the reference's rounding point; then double(n_t)^2 is added over all tensors in a
+// fixed order and the clip decision derived.  `seg` is the segment sums, in device memory or in LDS.
+template <typename SegPtr>
+__device__ __forceinline__ void decide_body(const ReduceArgs& a, SegPtr seg, double* lds_sum, int* lds_bad) {
+  double sq = 0.0;
   int bad = 0;
-  int i = threadIdx.x;
-  for (; i + kBlockThreads < a.n_tensors; i += 2 * kBlockThreads) {
-    const double v0 = a.tensor_sq[i], v1 = a.tensor_sq[i + kBlockThreads];
-    const int b0 = a.tensor_bad[i], b1 = a.tensor_bad[i + kBlockThreads];
-    s0 += v0; s1 += v1;
-    bad |= b0 | b1;
+  for (int t = threadIdx.x; t < a.n_tensors; t += kDecideThreads) {
+    const int b = a.tensor_seg_begin ? a.tensor_seg_begin[t] : 0;
+    const int e = a.tensor_seg_begin ? a.tensor_seg_begin[t + 1] : a.n_segments;
+    double sum = 0.0;
+    for (int i = b; i < e; i += 8) {
+      Partial w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) w[k] = seg[i + k < e ? i + k : e - 1];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if (i + k < e) {
+          sum += w[k].sumsq;
+          bad |= w[k].bad;
+        }
+      }
+    }
+    const float n = (float)sqrt(sum);
+    a.tensor_norm[t] = n;
+    sq += (double)n * (double)n;
   }
-  for (; i < a.n_tensors; i += kBlockThreads) {
-    s0 += a.tensor_sq[i];
-    bad |= a.tensor_bad[i];
-  }
-  double s = s0 + s1;
-  block_sum_or(s, bad, lds_sum, lds_bad);
+  block_sum_or<kDecideThreads / 64>(sq, bad, lds_sum, lds_bad);
   if (threadIdx.x == 0) {
     const int overflow = bad != 0 ? 1 : 0;
-    const double norm = sqrt(s);
+    const double norm = sqrt(sq);
     const double g = norm + 1e-6;
     const bool gate = overflow != 0 && a.ignore_overflow == 0;
     const bool clip = a.max_norm > 0.0f && !gate && (g > (double)a.max_norm);
+    const float coef = clip ? (float)((double)a.max_norm / g) : 1.0f;
     a.result->norm = norm;
-    a.result->coef = clip ? (float)((double)a.max_norm / g) : 1.0f;
+    a.result->coef = coef;
     a.result->overflow = overflow;
     a.result->clipped = clip ? 1 : 0;
     a.result->skipped = gate ? 1 : 0;
     if (a.result_copy != nullptr) {
       a.result_copy->norm = norm;
-      a.result_copy->coef = clip ? (float)((double)a.max_norm / g) : 1.0f;
+      a.result_copy->coef = coef;
       a.result_copy->overflow = overflow;
       a.result_copy->clipped = clip ? 1 : 0;
       a.result_copy->skipped = gate ? 1 : 0;
     }
   }
+}
+
+__global__ __launch_bounds__(kDecideThreads) void decide_kernel(ReduceArgs a) {
+  __shared__ double lds_sum[kDecideThreads / 64];
+  __shared__ int lds_bad[kDecideThreads / 64];
+  decide_body(a, a.seg_sums, lds_sum, lds_bad);
+}
+
+// Both stages in one block, for plans with few segments and partials: wavefront w adds segments
+// w, w + 16, ... (lane-strided, two loads in flight), the sums meet in LDS, and the block goes on
+// as decide_kernel does.  The segment sums are stored as well, for a later launch_decide.
+__global__ __launch_bounds__(kDecideThreads) void reduce_small_kernel(ReduceArgs a) {
+  __shared__ double lds_sum[kDecideThreads / 64];
+  __shared__ int lds_bad[kDecideThreads / 64];
+  __shared__ Partial seg_lds[kSmallReduceSegments];
+  const int lane = threadIdx.x & 63;
+  for (int seg = threadIdx.x >> 6; seg < a.n_segments; seg += kDecideThreads / 64) {
+    int64_t c0, c1;
+    segment_chunks(a, seg, c0, c1);
+    const int64_t end = c1 * a.partials_per_chunk;
+    int64_t i = c0 * a.partials_per_chunk + lane;
+    double s0 = 0.0, s1 = 0.0;
+    int bad = 0;
+    for (; i + 64 < end; i += 128) {
+      const Partial w0 = a.partials[i], w1 = a.partials[i + 64];
+      s0 += w0.sumsq; s1 += w1.sumsq;
+      bad |= w0.bad | w1.bad;
+    }
+    if (i < end) {
+      const Partial w = a.partials[i];
+      s0 += w.sumsq;
+      bad |= w.bad;
+    }
+    const double s = wave_total(s0 + s1);
+    bad = __any(bad) ? 1 : 0;
+    if (lane == 0) {
+      seg_lds[seg] = Partial{s, bad, 0};
+      a.seg_sums[seg] = Partial{s, bad, 0};
+    }
+  }
+  __syncthreads();
+  decide_body(a, &seg_lds[0], lds_sum, lds_bad);
 }
 
 __global__ __launch_bounds__(kBlockThreads) void fill_zero_kernel(char* p, int64_t nbytes) {
@@ -582,23 +613,22 @@ hipError_t launch_gated_pass(const PassArgs& a, bool streaming, hipStream_t stre
   return hipGetLastError();
 }
 
-hipError_t launch_finalize(const FinalizeArgs& a, hipStream_t stream) {
-  if (a.n_tensors > 0)
-    hipLaunchKernelGGL(finalize_tensors_kernel, dim3((unsigned)a.n_tensors), dim3(kBlockThreads), 0, stream, a);
-  hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
+hipError_t launch_reduce(const ReduceArgs& a, int64_t n_chunks, hipStream_t stream) {
+  if (a.n_segments <= kSmallReduceSegments && n_chunks * a.partials_per_chunk <= kSmallReducePartials) {
+    hipLaunchKernelGGL(reduce_small_kernel, dim3(1), dim3(kDecideThreads), 0, stream, a);
+    return hipGetLastError();
+  }
+  // one partial per chunk: a segment is a few hundred values; one per wavefront of every tile: thousands
+  if (a.partials_per_chunk > 1)
+    hipLaunchKernelGGL(reduce_segments_kernel<1024>, dim3((unsigned)a.n_segments), dim3(1024), 0, stream, a);
+  else
+    hipLaunchKernelGGL(reduce_segments_kernel<256>, dim3((unsigned)a.n_segments), dim3(256), 0, stream, a);
+  hipLaunchKernelGGL(decide_kernel, dim3(1), dim3(kDecideThreads), 0, stream, a);
   return hipGetLastError();
 }
 
-hipError_t launch_combine_tiles(const CombineArgs& a, hipStream_t stream) {
-  if (a.n_chunks <= 0) return hipSuccess;
-  const int per_block = kBlockThreads / 64;
-  hipLaunchKernelGGL(combine_tiles_kernel, dim3((unsigned)((a.n_chunks + per_block - 1) / per_block)), dim3(kBlockThreads), 0,
-                     stream, a);
-  return hipGetLastError();
-}
-
-hipError_t launch_finalize_total(const FinalizeArgs& a, hipStream_t stream) {
-  hipLaunchKernelGGL(finalize_total_kernel, dim3(1), dim3(kBlockThreads), 0, stream, a);
+hipError_t launch_decide(const ReduceArgs& a, hipStream_t stream) {
+  hipLaunchKernelGGL(decide_kernel, dim3(1), dim3(kDecideThreads), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -26,7 +26,8 @@ _is_contiguous = torch.Tensor.is_contiguous
 class _Steady:
     """What a group's last full step established, for the steps after it: as long as the same parameters all
     have contiguous gradients of the same dtype, a step is one pointer comparison per gradient and one launch."""
-    __slots__ = ("params_obj", "n", "param_ids", "table", "grad_ptrs", "grad_dtype", "steps_buf", "count", "device")
+    __slots__ = ("params_obj", "n", "param_ids", "table", "key", "grad_ptrs", "grad_dtype", "steps_buf", "count", "device",
+                 "param_ptr_ends")
 
 
 class _FusedBase(torch.optim.Optimizer):
@@ -62,6 +63,13 @@ class _FusedBase(torch.optim.Optimizer):
         self._tables.clear()
         self._steps.clear()
 
+    def invalidate_tables(self) -> None:
+        """Forget what earlier steps established about where parameters, gradients, state and model copies live.
+        For code that re-homes a parameter's ``.data`` (or a model copy) between steps: the next step then looks at
+        every tensor again and pushes all addresses to the device."""
+        self._steady.clear()
+        self._tables.clear()
+
     def _steady_grads(self, gi: int, group) -> Optional[Tuple["_Steady", List[torch.Tensor]]]:
         """The group's steady-state record and this step's gradients, or None when anything about the group
         differs from the step that made the record (then the full path runs and makes a new one)."""
@@ -76,12 +84,25 @@ class _FusedBase(torch.optim.Optimizer):
         for g in grads:
             if g is None:
                 return None
-        if grads[0].dtype != st.grad_dtype or grads[-1].dtype != st.grad_dtype or not all(map(_is_contiguous, grads)):
+        dt = st.grad_dtype
+        for g in grads:
+            if g.dtype != dt:
+                return None
+        if not all(map(_is_contiguous, grads)):
+            return None
+        # a parameter whose storage was replaced (``p.data = ...``) since the record was made: first and last are
+        # looked at here, code that re-homes others calls ``invalidate_tables``
+        if (params[0].data_ptr(), params[-1].data_ptr()) != st.param_ptr_ends:
             return None
         ptrs = list(map(_data_ptr, grads))
         if ptrs != st.grad_ptrs:
             st.table.update_pointers(grads=ptrs, stream=stream_handle(st.device))
             st.grad_ptrs = ptrs
+            # the full path's record of what the table points at must not outlive this re-pointing: a later
+            # full step with the old addresses would otherwise find them "unchanged" and skip the update
+            hit = self._tables.get(st.key)
+            if hit is not None and hit[0] is st.table:
+                self._tables[st.key] = (hit[0], (hit[1][0], tuple(ptrs)) + tuple(hit[1][2:]), hit[2])
         return st, grads
 
     def _make_steady(self, gi: int, group, table, grads: List[torch.Tensor], count: Optional[int]) -> None:
@@ -90,6 +111,8 @@ class _FusedBase(torch.optim.Optimizer):
         st.params_obj, st.n = params, len(params)
         st.param_ids = [id(p) for p in params]
         st.table = table
+        st.key = table.cache_key
+        st.param_ptr_ends = (params[0].data_ptr(), params[-1].data_ptr())
         st.grad_ptrs = [g.data_ptr() for g in grads]
         st.grad_dtype = grads[0].dtype
         st.device = params[0].device
@@ -162,6 +185,7 @@ class _FusedBase(torch.optim.Optimizer):
         # live until the launch that reads them is queued (their memory is reused in stream order) and whose
         # release lets the next backward find the same addresses free
         self._tables[key] = (table, ptrs, [params, state1, state2, copies])
+        table.cache_key = key
         return table
 
 

@@ -125,6 +125,13 @@ class TensorPlan:
         the stream: call it once, right after building a plan whose destinations hold nothing yet."""
         return self.plan.tune(self._stream())
 
+    def write_order(self) -> int:
+        return self.plan.write_order
+
+    def set_write_order(self, order: int) -> None:
+        """Use an order measured earlier (on a table of the same layout) instead of measuring again."""
+        self.plan.set_write_order(order)
+
     def repoint_sources(self, src_ptrs: Sequence[int]) -> None:
         """New source addresses (one per tensor, same sizes and dtypes, contiguous) without any per-tensor check:
         for callers that have established those facts themselves."""
@@ -179,6 +186,9 @@ class TensorPlan:
 
     def close(self) -> None:
         self.plan.close()
+
+    def is_open(self) -> bool:
+        return self.plan.is_open()
 
 
 def fill_zero_(t: torch.Tensor) -> torch.Tensor:

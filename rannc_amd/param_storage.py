@@ -57,6 +57,7 @@ class _PlanCache:
         self._plan: Optional[TensorPlan] = None
         self._token = None
         self._src_ptrs: Optional[List[int]] = None
+        self._orders: Dict[tuple, int] = {}       # layout (sizes and dtypes) -> write order measured for it
 
     def get_same_shapes(self, token, srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor],
                         tune_new: bool = False) -> TensorPlan:
@@ -102,7 +103,13 @@ class _PlanCache:
             self._plan.close()
         self._plan = TensorPlan(srcs, dsts)
         if tune_new and dsts is not None:
-            self._plan.tune()
+            # measured once per layout: a table rebuilt for the same sizes and dtypes takes the order found then,
+            # so that its destinations are not overwritten by another measurement
+            layout = (tuple(k[1:] for k in key[0]), tuple(k[1:] for k in key[1]))
+            if layout in self._orders:
+                self._plan.set_write_order(self._orders[layout])
+            else:
+                self._orders[layout] = self._plan.tune()
         self._key = key
         return self._plan
 

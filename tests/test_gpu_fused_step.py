@@ -204,38 +204,40 @@ def test_repeatable_bits():
     assert_bits_equal(a[2], b[2], "run-to-run")
 
 
-@pytest.mark.parametrize("env", [
-    {"RG_XCD_REDUCE": "-1"}, {"RG_XCD_REDUCE": "3", "RG_XCD_WRITE": "5"}, {"RG_XCD_WRITE": "-1"},
-    {"RG_WRITE_TILE_ELEMS": "256"}, {"RG_WRITE_TILE_ELEMS": "4096", "RG_REDUCE_TILE_FACTOR": "4"},
-    {"RG_REDUCE_TILE_FACTOR": "1"},
-])
-def test_tuning_knobs_do_not_change_results(env, monkeypatch):
-    """Block -> XCD mappings and tile sizes only reorder the work: values are bit-identical, sums
-    within the norm tolerance (their order changes with the tile size)."""
+@pytest.mark.parametrize("order", [0, 3, 64, 256, -1])
+def test_every_write_order_gives_the_oracles_bits(order):
+    """The order in which a writing pass hands its tiles to the XCDs (``rg_plan_set_write_order``, what
+    ``rg_plan_tune`` chooses between) only reorders the work: with each order the two-pass step and the one-pass
+    ``unscale_pack`` are held to the CPU oracle - bucket bit-exact, norms and coefficient to 1e-6."""
     g = torch.Generator().manual_seed(77)
-    cpu = [(torch.randn(n, generator=g) * 8).to(torch.bfloat16) for n in (100003, 5, 16384, 40000, 1, 262147)]
-    srcs = [t.to("cuda:0") for t in cpu]
-    ref_out = [torch.zeros(t.shape, device="cuda:0") for t in cpu]
-    ref = TensorPlan(srcs, ref_out, chunk_elems=4096)
-    ref.fused_step(0.125, 0.5)
-    want = ref.result()
-    ref_pack = [torch.zeros(t.shape, device="cuda:0") for t in cpu]
-    rp = TensorPlan(srcs, ref_pack, chunk_elems=4096)
-    rp.unscale_pack(0.125)
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
-    out = [torch.full(t.shape, 3.0, device="cuda:0") for t in cpu]
-    plan = TensorPlan(srcs, out, chunk_elems=4096)           # the knobs are read when the plan is created
+    grads = [(torch.randn(n, generator=g) * 8).to(torch.bfloat16) for n in (100003, 5, 16384, 40000, 1, 262147)]
+    srcs = place_in_arena(grads, DEV, 1, 3)
+    total = sum(t.numel() for t in grads)
+    offs, _ = oracle.bucket_layout([t.numel() for t in grads], ["f32"] * len(grads))
+    bucket = torch.full((total + 1,), 3.0, device=DEV)[1:]
+    dsts = [bucket.narrow(0, o, t.numel()) for o, t in zip(offs, grads)]
+    plan = TensorPlan(srcs, dsts, chunk_elems=4096)
+    plan.set_write_order(order)
+    assert plan.write_order() == order
     plan.fused_step(0.125, 0.5)
-    got = plan.result()
-    assert (got.overflow, got.clipped) == (want.overflow, want.clipped) and got.clipped == 1
-    assert got.norm == want.norm and got.coef == want.coef       # the read pass keeps its chunk partials whatever the mapping
-    for a, b in zip(out, ref_out):
-        assert_bits_equal(a.cpu(), b.cpu(), f"fused step with {env}")
+    res, tn = plan.result(), plan.tensor_norms()
+    want = _check_against_oracle(grads, "f32", 0.125, 0.5, res, tn, bucket.cpu())
+    assert want.coef is not None
+    bucket.fill_(3.0)
     plan.unscale_pack(0.125)
-    assert math.isclose(plan.result().norm, rp.result().norm, rel_tol=1e-12)
-    for a, b in zip(out, ref_pack):
-        assert_bits_equal(a.cpu(), b.cpu(), f"unscale_pack with {env}")
+    res, tn = plan.result(), plan.tensor_norms()
+    _check_against_oracle(grads, "f32", 0.125, math.inf, res, tn, bucket.cpu())
+    plan.close()
+
+
+def test_set_write_order_rejects_values_outside_its_range():
+    t = torch.zeros(4096, device=DEV)
+    plan = TensorPlan([t], [torch.zeros_like(t)])
+    with pytest.raises(ValueError, match="order"):
+        plan.set_write_order(-2)
+    with pytest.raises(ValueError, match="order"):
+        plan.set_write_order(1 << 20)
+    plan.close()
 
 
 # ----------------------------------------------------------------------------- one-pass strategy

@@ -680,3 +680,40 @@ def test_amp_master_params_completes_a_deferred_write():
     want, _ = oracle.unscale_and_check(grads, 1.0 / 256.0)
     for m, w in zip(masters, want):
         assert_bits_equal(m.grad.cpu(), w, "master gradient handed out by master_params")
+
+
+@pytest.mark.parametrize("reader", ["named_master_params", "zip_params"])
+def test_amp_named_master_params_completes_a_deferred_write(reader):
+    """The reference's own tests read the unscaled gradients as ``p.grad for n, p in named_master_params(...)``
+    (``test/common.py:86``): right after ``scale_loss`` exits - on the first step and after a step that clipped,
+    when the default fused mode has deferred the write - that must hand out what a ``fused=False`` run holds."""
+    def run(fused):
+        torch.manual_seed(11)
+        model = _tiny_model()
+        opt = torch.optim.SGD(model.parameters(), lr=0.0)
+        model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, fused=fused)
+        rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+        gen = torch.Generator().manual_seed(3)
+        seen = []
+        for step in range(3):
+            x = torch.randn(16, 32, generator=gen).to(DEV, torch.float16)
+            loss = rm(x).float().pow(2).mean()
+            with amp.scale_loss(loss, opt) as scaled:
+                scaled.backward()
+            if fused and step != 1:
+                assert opt._amp_stash.pending_finish          # step 0, and step 2 (step 1 clipped): write deferred
+            if reader == "named_master_params":
+                grads = [p.grad.detach().cpu().clone() for _, p in amp.named_master_params(model, opt)]
+            else:
+                grads = [m.grad.detach().cpu().clone() for m, _ in amp.zip_params(opt)]
+            assert not opt._amp_stash.pending_finish
+            seen.append(grads)
+            rm.clip_grad_norm(1e9 if step == 0 else 1e-3)     # steps 1 and 2 clip
+            opt.step()
+            opt.zero_grad()
+        return seen
+    got, want = run(True), run(False)
+    for step, (gs, ws) in enumerate(zip(got, want)):
+        assert len(gs) == len(ws) > 0
+        for g, w in zip(gs, ws):
+            assert_bits_equal(g, w, f"master gradient read through {reader} at step {step}")

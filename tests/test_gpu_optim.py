@@ -354,3 +354,51 @@ def test_optimizer_step_on_a_tensor_beyond_two_to_the_31_elements():
         for lo in range(0, n, step):                     # every element, slice by slice
             hi = min(n, lo + step)
             torch.testing.assert_close(p[lo:hi], before[lo:hi] - 0.25 * g[lo:hi], rtol=2e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("fused_cls,kw", [(FusedAdam, dict(lr=1e-2)), (FusedSGD, dict(lr=0.05, momentum=0.9))])
+def test_gradients_that_move_away_and_back_are_followed(fused_cls, kw):
+    """Gradients at addresses A (full step), at B (steady step: the device table is re-pointed), one step with a
+    missing gradient (full path again), then all gradients back at A: the table must read A, not the B it was last
+    pointed at.  Compared step by step with a twin optimizer that is handed the same values in fresh tensors."""
+    torch.manual_seed(3)
+    shapes = [(257,), (64, 33), (5,)]
+    params = [torch.nn.Parameter(torch.randn(s, device=DEV)) for s in shapes]
+    twins = [torch.nn.Parameter(p.detach().clone()) for p in params]
+    opt, ref = fused_cls(params, **kw), fused_cls(twins, **kw)
+    set_a = [torch.randn(s, device=DEV) for s in shapes]
+    set_b = [torch.randn(s, device=DEV) for s in shapes]
+    plan = [(set_a, None), (set_a, None), (set_b, None), (set_b, 1), (set_a, None), (set_a, None)]
+    for step, (grads, missing) in enumerate(plan):
+        for i, (p, t, g) in enumerate(zip(params, twins, grads)):
+            g.normal_()                                           # new values at the same addresses
+            p.grad = None if i == missing else g
+            t.grad = None if i == missing else g.clone()          # the twin always sees fresh tensors
+        if step == 3:
+            ref.invalidate_tables()
+        opt.step()
+        ref.step()
+        for i, (p, t) in enumerate(zip(params, twins)):
+            assert_bits_equal(p.detach(), t.detach(), f"param {i} after step {step}")
+
+
+def test_invalidate_tables_after_rehoming_a_parameter():
+    """A parameter whose storage is replaced between steps (``p.data = ...``, what the offload wrapper and
+    ``_sync_orig_params`` do) is followed once ``invalidate_tables`` has been called."""
+    torch.manual_seed(4)
+    params = [torch.nn.Parameter(torch.randn(s, device=DEV)) for s in ((100,), (33, 7), (4096,))]
+    twins = [torch.nn.Parameter(p.detach().clone()) for p in params]
+    opt, ref = FusedAdam(params, lr=1e-2), FusedAdam(twins, lr=1e-2)
+    grads = [torch.randn(p.shape, device=DEV) for p in params]
+    for step in range(4):
+        for p, t, g in zip(params, twins, grads):
+            g.normal_()
+            p.grad, t.grad = g, g.clone()
+        if step == 2:
+            with torch.no_grad():
+                params[1].data = params[1].data.clone()           # middle parameter: not seen by the first / last check
+            opt.invalidate_tables()
+        opt.step()
+        ref.step()
+        for i, (p, t) in enumerate(zip(params, twins)):
+            assert_bits_equal(p.detach(), t.detach(), f"param {i} after step {step}")

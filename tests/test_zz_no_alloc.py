@@ -75,6 +75,19 @@ def test_static_step_matches_the_plan_twice_in_a_row_second_call_smaller():
     assert r.overflow == 1
 
 
+def test_static_step_fp32_sources_large_enough_for_the_largest_chunks():
+    """fp32 sources switch to chunks of 8192 elements (32 KiB of source, as for 16-bit types) once the tensor is
+    large enough for the cap to bind - above about 16.8 M elements; the one-tensor plan does the same, and norm,
+    coefficient and every written bit must still agree."""
+    dev = torch.device("cuda", 0)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    r = _case(35_000_003, torch.float32, torch.float32, 1, 2.0 ** -8, 1.0, dev, gen)
+    assert r.clipped == 1
+    r = _case(20_000_001, torch.float32, torch.float16, 0, 2.0 ** -8, 1.0, dev, gen)
+    assert r.clipped == 1
+    _case(9_000_000, torch.float32, torch.bfloat16, 2, 2.0 ** -8, 1e9, dev, gen)     # smaller again, no clip
+
+
 def test_static_step_in_place_clip():
     dev = torch.device("cuda", 0)
     gen = torch.Generator(device=dev).manual_seed(6)
@@ -90,8 +103,12 @@ def test_static_step_in_place_clip():
 def test_static_step_rejects_what_it_cannot_hold():
     dev = torch.device("cuda", 0)
     t = torch.zeros(8, device=dev)
+    # the limit is 8 GiB of source: 2^32 elements of a 16-bit type, 2^31 of fp32
     with pytest.raises(ValueError, match="exceed the limit"):
-        _lib.fused_step_static(t.data_ptr(), t.data_ptr(), _lib.RG_STATIC_MAX_NUMEL + 1, _lib.RG_F32, _lib.RG_F32,
+        _lib.fused_step_static(t.data_ptr(), t.data_ptr(), _lib.RG_STATIC_MAX_NUMEL + 1, _lib.RG_F16, _lib.RG_F16,
+                               1.0, 1.0, 0, None, 0, 0)
+    with pytest.raises(ValueError, match="exceed the limit"):
+        _lib.fused_step_static(t.data_ptr(), t.data_ptr(), _lib.RG_STATIC_MAX_NUMEL // 2 + 1, _lib.RG_F32, _lib.RG_F32,
                                1.0, 1.0, 0, None, 0, 0)
     with pytest.raises(ValueError, match="inv_scale"):
         _lib.fused_step_static(t.data_ptr(), t.data_ptr(), 8, _lib.RG_F32, _lib.RG_F32, 0.0, 1.0, 0, None, 0, 0)
