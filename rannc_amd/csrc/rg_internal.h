@@ -112,7 +112,7 @@ constexpr int kWaveSlotsPerTile = kWriteThreads / 64;   // partials one tile of 
 // per segment adds its partials in a fixed order, then a single block adds each tensor's segment sums (one thread
 // per tensor), rounds to n_t = float(sqrt(sum)), adds double(n_t)^2 over the tensors and takes the clip decision.
 // Plans with few segments and partials run both stages in that single block: one launch.
-constexpr int64_t kSegmentChunks = 256;
+constexpr int64_t kSegmentChunks = 64;
 constexpr int kMaxSegmentsPerTensor = 64;
 constexpr int kDecideThreads = 1024;
 constexpr int kSmallReduceSegments = 64;        // the one-launch form: at most this many segments ...

@@ -427,7 +427,7 @@ __device__ __forceinline__ void segment_chunks(const ReduceArgs& a, int seg, int
   }
 }
 
-// Stage 1: block b adds the partials of segment b (thread-strided with four independent loads in
+// Stage 1: block b adds the partials of segment b (thread-strided with eight independent loads in
 // flight, then a fixed tree).
 template <int THREADS>
 __global__ __launch_bounds__(THREADS) void reduce_segments_kernel(ReduceArgs a) {
@@ -437,22 +437,26 @@ __global__ __launch_bounds__(THREADS) void reduce_segments_kernel(ReduceArgs a) 
   segment_chunks(a, (int)blockIdx.x, c0, c1);
   const int64_t end = c1 * a.partials_per_chunk;
   int64_t i = c0 * a.partials_per_chunk + threadIdx.x;
-  double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+  double s[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
   int bad = 0;
-  for (; i + 3 * THREADS < end; i += 4 * THREADS) {
-    const Partial w0 = a.partials[i], w1 = a.partials[i + THREADS];
-    const Partial w2 = a.partials[i + 2 * THREADS], w3 = a.partials[i + 3 * THREADS];
-    s0 += w0.sumsq; s1 += w1.sumsq; s2 += w2.sumsq; s3 += w3.sumsq;
-    bad |= w0.bad | w1.bad | w2.bad | w3.bad;
+  for (; i < end; i += 8 * THREADS) {
+    Partial w[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t j = i + (int64_t)k * THREADS;
+      w[k] = a.partials[j < end ? j : end - 1];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (i + (int64_t)k * THREADS < end) {
+        s[k] += w[k].sumsq;
+        bad |= w[k].bad;
+      }
+    }
   }
-  for (; i < end; i += THREADS) {
-    const Partial w = a.partials[i];
-    s0 += w.sumsq;
-    bad |= w.bad;
-  }
-  double s = (s0 + s1) + (s2 + s3);
-  block_sum_or<THREADS / 64>(s, bad, lds_sum, lds_bad);
-  if (threadIdx.x == 0) a.seg_sums[blockIdx.x] = Partial{s, bad, 0};
+  double total = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+  block_sum_or<THREADS / 64>(total, bad, lds_sum, lds_bad);
+  if (threadIdx.x == 0) a.seg_sums[blockIdx.x] = Partial{total, bad, 0};
 }
 
 // Stage 2, one block: thread t adds the segment sums of tensor t in order (eight loads in flight) and rounds
@@ -512,7 +516,7 @@ __global__ __launch_bounds__(kDecideThreads) void decide_kernel(ReduceArgs a) {
 }
 
 // Both stages in one block, for plans with few segments and partials: wavefront w adds segments
-// w, w + 16, ... (lane-strided, two loads in flight), the sums meet in LDS, and the block goes on
+// w, w + 16, ... (lane-strided, four loads in flight), the sums meet in LDS, and the block goes on
 // as decide_kernel does.  The segment sums are stored as well, for a later launch_decide.
 __global__ __launch_bounds__(kDecideThreads) void reduce_small_kernel(ReduceArgs a) {
   __shared__ double lds_sum[kDecideThreads / 64];
@@ -524,19 +528,21 @@ __global__ __launch_bounds__(kDecideThreads) void reduce_small_kernel(ReduceArgs
     segment_chunks(a, seg, c0, c1);
     const int64_t end = c1 * a.partials_per_chunk;
     int64_t i = c0 * a.partials_per_chunk + lane;
-    double s0 = 0.0, s1 = 0.0;
+    double s4[4] = {0.0, 0.0, 0.0, 0.0};
     int bad = 0;
-    for (; i + 64 < end; i += 128) {
-      const Partial w0 = a.partials[i], w1 = a.partials[i + 64];
-      s0 += w0.sumsq; s1 += w1.sumsq;
-      bad |= w0.bad | w1.bad;
+    for (; i < end; i += 256) {
+      Partial w[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) w[k] = a.partials[i + 64 * k < end ? i + 64 * k : end - 1];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (i + 64 * k < end) {
+          s4[k] += w[k].sumsq;
+          bad |= w[k].bad;
+        }
+      }
     }
-    if (i < end) {
-      const Partial w = a.partials[i];
-      s0 += w.sumsq;
-      bad |= w.bad;
-    }
-    const double s = wave_total(s0 + s1);
+    const double s = wave_total((s4[0] + s4[1]) + (s4[2] + s4[3]));
     bad = __any(bad) ? 1 : 0;
     if (lane == 0) {
       seg_lds[seg] = Partial{s, bad, 0};
@@ -618,11 +624,7 @@ hipError_t launch_reduce(const ReduceArgs& a, int64_t n_chunks, hipStream_t stre
     hipLaunchKernelGGL(reduce_small_kernel, dim3(1), dim3(kDecideThreads), 0, stream, a);
     return hipGetLastError();
   }
-  // one partial per chunk: a segment is a few hundred values; one per wavefront of every tile: thousands
-  if (a.partials_per_chunk > 1)
-    hipLaunchKernelGGL(reduce_segments_kernel<1024>, dim3((unsigned)a.n_segments), dim3(1024), 0, stream, a);
-  else
-    hipLaunchKernelGGL(reduce_segments_kernel<256>, dim3((unsigned)a.n_segments), dim3(256), 0, stream, a);
+  hipLaunchKernelGGL(reduce_segments_kernel<256>, dim3((unsigned)a.n_segments), dim3(256), 0, stream, a);
   hipLaunchKernelGGL(decide_kernel, dim3(1), dim3(kDecideThreads), 0, stream, a);
   return hipGetLastError();
 }
