@@ -79,6 +79,33 @@ template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
   else *g = v;
 }
 
+// Stores whose order in the instruction stream is fixed (volatile asm statements keep their relative order):
+// st16_ordered is a plain 16-byte store, st16_last / st8_last are the stores above issued after it.
+__device__ __forceinline__ void st16_ordered(char* p, u32x4 v) {
+  RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
+  asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(g), "v"(v));
+}
+template <bool NT> __device__ __forceinline__ void st16_last(char* p, u32x4 v) {
+  RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
+#ifdef RG_STREAM_STORE_BITS
+  if (NT) asm volatile("global_store_dwordx4 %0, %1, off " RG_STREAM_STORE_BITS : : "v"(g), "v"(v));
+  else asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(g), "v"(v));
+#else
+  if (NT) asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(g), "v"(v));
+  else asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(g), "v"(v));
+#endif
+}
+template <bool NT> __device__ __forceinline__ void st8_last(char* p, u32x2 v) {
+  RG_GLOBAL u32x2_a2* g = (RG_GLOBAL u32x2_a2*)p;
+#ifdef RG_STREAM_STORE_BITS
+  if (NT) asm volatile("global_store_dwordx2 %0, %1, off " RG_STREAM_STORE_BITS : : "v"(g), "v"(v));
+  else asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(g), "v"(v));
+#else
+  if (NT) asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(g), "v"(v));
+  else asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(g), "v"(v));
+#endif
+}
+
 template <int DT, int E, bool NT> struct Mem;
 template <bool NT> struct Mem<RG_F32, 4, NT> {
   static __device__ __forceinline__ Raw<RG_F32, 4> load(const char* p) { return {ld16_a4<NT>(p)}; }
@@ -217,6 +244,22 @@ __device__ __forceinline__ double wave_total(double x) {
   x += dpp_row_shr<4>(x);
   x += dpp_row_shr<8>(x);
   return (read_lane(x, 15) + read_lane(x, 31)) + (read_lane(x, 47) + read_lane(x, 63));
+}
+
+// Sum of one float per lane over the wavefront in six DPP additions (two butterflies inside each quad, two row
+// shifts, two row broadcasts: ((r3 + r2) + (r1 + r0)) of the row sums ends up in lane 63), returned to every lane.
+// All 64 lanes must be active.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_f32(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_total_f32(float x) {
+  x += dpp_f32<0xb1, 0xf>(x);    // quad_perm:[1,0,3,2]
+  x += dpp_f32<0x4e, 0xf>(x);    // quad_perm:[2,3,0,1]
+  x += dpp_f32<0x114, 0xf>(x);   // row_shr:4
+  x += dpp_f32<0x118, 0xf>(x);   // row_shr:8
+  x += dpp_f32<0x142, 0xa>(x);   // row_bcast:15 into rows 1 and 3
+  x += dpp_f32<0x143, 0xc>(x);   // row_bcast:31 into rows 2 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
 }
 
 }  // namespace

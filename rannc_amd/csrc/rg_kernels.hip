@@ -40,9 +40,29 @@ template <int MODE> struct PassThreads { static constexpr int value = (MODE & kM
 // coef is 1 when nothing is clipped: v * 1 is v bit for bit, so no branch is needed.
 // The two multiplies are never fused or reassociated (the file is built with
 // -ffp-contract=off), so the result matches `x.float() * inv_scale` then `mul_(coef)`.
+// A vector store that process_chunk holds back for its caller (bytes == 0: none).
+struct PendingStore {
+  u32x4 v;
+  char* p;
+  int bytes;
+};
+
+#ifndef RG_DEFER_LAST_STORE
+#define RG_DEFER_LAST_STORE 1
+#endif
+// A pass that sums while it writes ends every wavefront with a store that depends on everything before it: the
+// record of its partial sum.  Measured on MI355X, that trailing store costs such a pass 4-5 % whatever its size,
+// cache policy or address (a record stored in mid-life, or none at all, costs nothing: the time goes into the end
+// of blocks that live under 4 us).  With fp32 sources most of it comes back when the last vector store is held
+// back until the record has been issued - the caller reduces, stores the record, then the held vector - (+5-7 %
+// for fp32 -> fp32 / bf16 / fp16); with 16-bit sources the same reordering loses 2 %, so they keep the plain order.
+template <int S, int MODE> struct DefersLastStore {
+  static constexpr bool value = RG_DEFER_LAST_STORE && S == RG_F32 && (MODE & kModeReduce) != 0 && (MODE & kModeWrite) != 0;
+};
+
 template <int S, int D, int MODE, bool NT, int T = PassThreads<MODE>::value, bool HEAD = true>
 __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len, float scale, float coef,
-                                              bool raw_copy, float (&acc)[8]) {
+                                              bool raw_copy, float (&acc)[8], PendingStore& pending) {
   constexpr int SS = ElemSize<S>::value;
   constexpr int DS = ElemSize<D>::value;
   constexpr bool kWrite = (MODE & kModeWrite) != 0;
@@ -107,7 +127,8 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   // previous destination values, only when accumulating (the type does not exist otherwise)
   struct Nothing {};
   using Old = std::conditional_t<kAcc, Raw<kAcc ? D : S, E>, Nothing>;
-  auto consume = [&](const Raw<S, E>& in, const Old* old, int e, bool valid) {
+  constexpr bool kDefer = DefersLastStore<S, MODE>::value;
+  auto consume = [&](const Raw<S, E>& in, const Old* old, int e, bool valid, bool hold) {
     bool copied = false;
     if constexpr (S == D && kWrite) {
       if (raw_copy) {
@@ -132,7 +153,21 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
         if (kWrite) f[j] = round_dst<D>(v * coef);
       }
       if constexpr (kWrite) {
-        if (valid) Mem<D, E, NT>::store(db + (size_t)e * DS, Codec<D, E>::pack(f));
+        if constexpr (kDefer) {
+          if (hold) {
+            if (valid) {
+              const Raw<D, E> out = Codec<D, E>::pack(f);
+              if constexpr (sizeof(out.v) == 16) pending.v = out.v;
+              else pending.v = u32x4{out.v[0], out.v[1], 0u, 0u};
+              pending.p = db + (size_t)e * DS;
+              pending.bytes = (int)sizeof(out.v);
+            }
+          } else if (valid) {
+            Mem<D, E, NT>::store(db + (size_t)e * DS, Codec<D, E>::pack(f));
+          }
+        } else {
+          if (valid) Mem<D, E, NT>::store(db + (size_t)e * DS, Codec<D, E>::pack(f));
+        }
       }
     }
   };
@@ -147,8 +182,10 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
 #pragma unroll
       for (int u = 0; u < U; ++u) old[u] = Mem<D, E, NT>::load(db + (size_t)(base + (u * T + tid) * E) * DS);
     }
+    // the last vector store of the chunk is the one held back (only its final instruction: u == U - 1)
+    const bool final_iter = kDefer && base + kIter == nbody;
 #pragma unroll
-    for (int u = 0; u < U; ++u) consume(in[u], &old[kAcc ? u : 0], base + (u * T + tid) * E, true);
+    for (int u = 0; u < U; ++u) consume(in[u], &old[kAcc ? u : 0], base + (u * T + tid) * E, true, final_iter && u == U - 1);
   }
   if (base < nbody) {
     // Last, partial iteration: lanes past the end re-read the final vector (an address that
@@ -164,7 +201,7 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int e = base + (u * T + tid) * E;
-      consume(in[u], &old[kAcc ? u : 0], e, e < nbody);
+      consume(in[u], &old[kAcc ? u : 0], e, e < nbody, kDefer && u == U - 1);
     }
   }
 
@@ -258,13 +295,14 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
   const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale == 1.0f;   // never when accumulating
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  PendingStore pending{u32x4{0u, 0u, 0u, 0u}, nullptr, 0};
   if (sp == nullptr || a.zero_fill) {
     if constexpr ((MODE & kModeAccumulate) != 0) {
       // Nothing to add: the destination keeps its values, which still count towards the norm.
       if constexpr ((MODE & kModeReduce) != 0) {
-        if (dst_kind == RG_F32) process_chunk<RG_F32, RG_F32, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
-        else if (dst_kind == RG_F16) process_chunk<RG_F16, RG_F16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
-        else process_chunk<RG_BF16, RG_BF16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
+        if (dst_kind == RG_F32) process_chunk<RG_F32, RG_F32, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc, pending);
+        else if (dst_kind == RG_F16) process_chunk<RG_F16, RG_F16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc, pending);
+        else process_chunk<RG_BF16, RG_BF16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc, pending);
       }
     } else if (MODE & kModeWrite) {
       zero_range<NT, T, PEEL>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
@@ -277,8 +315,8 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
     const bool has_head = ((MODE & kModeWrite) == 0 || PEEL) && (peeled & (peel - 1)) != 0;
 #define RG_PAIR(S, D)                                                                         \
   case S * 3 + D:                                                                             \
-    if (has_head) process_chunk<S, D, MODE, NT, T, true>(sp, dp, len, a.scale, coef, raw_copy, acc);  \
-    else process_chunk<S, D, MODE, NT, T, false>(sp, dp, len, a.scale, coef, raw_copy, acc);  \
+    if (has_head) process_chunk<S, D, MODE, NT, T, true>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);  \
+    else process_chunk<S, D, MODE, NT, T, false>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);  \
     break;
     switch (src_kind * 3 + dst_kind) {
       RG_PAIR(RG_F32, RG_F32)
@@ -290,28 +328,22 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
       RG_PAIR(RG_BF16, RG_F32)
       RG_PAIR(RG_BF16, RG_F16)
       default:
-        if (has_head) process_chunk<RG_BF16, RG_BF16, MODE, NT, T, true>(sp, dp, len, a.scale, coef, raw_copy, acc);
-        else process_chunk<RG_BF16, RG_BF16, MODE, NT, T, false>(sp, dp, len, a.scale, coef, raw_copy, acc);
+        if (has_head) process_chunk<RG_BF16, RG_BF16, MODE, NT, T, true>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);
+        else process_chunk<RG_BF16, RG_BF16, MODE, NT, T, false>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);
         break;
     }
 #undef RG_PAIR
   }
 
   if (MODE & kModeReduce) {
-    // Fixed-order combine: 8 sums of the thread, 64 lanes of the wavefront by DPP row scans.
-    // Everything past the per-thread fp32 sums is double.
-    // A non-finite input makes its square, and so the sum, non-finite; a finite sum therefore
-    // proves every input was finite.  Only when a sum is not finite are the elements looked
-    // at again one by one (the sum can also overflow from finite inputs).
+    // Fixed-order combine.  A non-finite input makes its square, and so the sum, non-finite; a finite sum
+    // therefore proves every input was finite.  Only when a sum is not finite are the elements looked at again
+    // one by one (the sum can also overflow from finite inputs).
     constexpr int kWaves = T / 64;
-    double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
-               (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
-    s = wave_total(s);
     if constexpr (kWavePartials) {
-      // One partial per wavefront.  A wavefront whose sum is not finite looks at every element
-      // of the tile again (its own elements are strided through it), 64 at a time.
-      int bad = 0;
-      if (!(fabs(s) <= 1.79769313486231570e308)) {
+      // One partial per wavefront: sum and flag leave in one 16-byte store.  A wavefront whose sum is not finite
+      // looks at every element of the tile again (its own elements are strided through it), 64 at a time.
+      auto rescan = [&]() -> int {
         int mine = 0;
         if (sp != nullptr) {
           const int lane = threadIdx.x & 63;
@@ -322,12 +354,34 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
                                                                                         : nonfinite_at<RG_BF16>(q)) ? 1 : 0;
           }
         }
-        bad = __any(mine) ? 1 : 0;
+        return __any(mine) ? 1 : 0;
+      };
+      Partial* const slot = &a.partials[slot_id * kSlots + (threadIdx.x >> 6)];
+      if (RG_DEFER_LAST_STORE && src_kind == RG_F32 && sp != nullptr) {
+        // process_chunk held the last vector store back, and that store now waits for the record.  The 8 elements
+        // of a lane and the 64 lanes are therefore added in fp32 (six DPP additions in a fixed order): 512 squares
+        // summed as a tree are within a few 1e-8 of their exact sum, and everything after the record is double.
+        const float lane_sum = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+        const float total = wave_total_f32(lane_sum);
+        const int bad = !(fabsf(total) <= 3.40282346638528859812e38f) ? rescan() : 0;
+        // the record, then the held vector: both through volatile asm, which keeps their order
+        const Partial rec{(double)total, bad, 0};
+        if ((threadIdx.x & 63) == 0) st16_ordered(reinterpret_cast<char*>(slot), __builtin_bit_cast(u32x4, rec));
+        if (pending.bytes == 16) st16_last<NT>(pending.p, pending.v);
+        else if (pending.bytes == 8) st8_last<NT>(pending.p, u32x2{pending.v[0], pending.v[1]});
+      } else {
+        double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
+                   (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
+        s = wave_total(s);
+        const int bad = !(fabs(s) <= 1.79769313486231570e308) ? rescan() : 0;
+        if ((threadIdx.x & 63) == 0) *slot = Partial{s, bad, 0};
       }
-      // sum and flag leave in one 16-byte store
-      if ((threadIdx.x & 63) == 0) a.partials[slot_id * kSlots + (threadIdx.x >> 6)] = Partial{s, bad, 0};
     } else {
-      // One partial per block, the wavefronts combined through LDS in index order.
+      // One partial per block: the 8 sums of the thread, the 64 lanes of the wavefront by DPP row scans, the
+      // wavefronts through LDS in index order.  Everything past the per-thread fp32 sums is double.
+      double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
+                 (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
+      s = wave_total(s);
       __shared__ double wave_sum[kWaves];
       if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = s;
       __syncthreads();
