@@ -18,7 +18,7 @@ __device__ __forceinline__ u32x4 as_u32x4(f32x4 v) { return __builtin_bit_cast(u
 // Streaming store with the cache policy of the passes that write one stream per launch.
 __device__ __forceinline__ void st16_stream(char* p, u32x4 v) {
   RG_GLOBAL u32x4* g = (RG_GLOBAL u32x4*)p;
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(g), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(g), "v"(v) : "memory");   // two wait states: the compiler does not know this is a 128-bit store whose data registers must not be overwritten yet
 }
 
 // Read only: the read-only pass's shape.  256 threads, eight 16-byte nontemporal loads in flight per

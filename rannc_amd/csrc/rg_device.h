@@ -56,11 +56,16 @@ template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
 #ifndef RG_NT_STORES
 #define RG_NT_STORES 1
 #endif
+// gfx940-family hazard: a VALU instruction that overwrites the data registers of a store of more than 64 bits
+// within two wait states of it changes what is stored.  The compiler spaces its own stores accordingly, but it
+// does not know that an asm statement is a store, so every 128-bit store issued through asm brings its own two
+// wait states (the 64-bit ones are not affected).
+#define RG_STORE_HAZARD_NOP "\n\ts_nop 1"
 template <bool NT> __device__ __forceinline__ void st16(char* p, u32x4 v) {
   RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
 #ifdef RG_STREAM_STORE_BITS
   if (NT) {
-    asm volatile("global_store_dwordx4 %0, %1, off " RG_STREAM_STORE_BITS : : "v"(g), "v"(v));
+    asm volatile("global_store_dwordx4 %0, %1, off " RG_STREAM_STORE_BITS RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
     return;
   }
 #endif
@@ -83,16 +88,16 @@ template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
 // st16_ordered is a plain 16-byte store, st16_last / st8_last are the stores above issued after it.
 __device__ __forceinline__ void st16_ordered(char* p, u32x4 v) {
   RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
-  asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(g), "v"(v));
+  asm volatile("global_store_dwordx4 %0, %1, off" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
 }
 template <bool NT> __device__ __forceinline__ void st16_last(char* p, u32x4 v) {
   RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
 #ifdef RG_STREAM_STORE_BITS
-  if (NT) asm volatile("global_store_dwordx4 %0, %1, off " RG_STREAM_STORE_BITS : : "v"(g), "v"(v));
-  else asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(g), "v"(v));
+  if (NT) asm volatile("global_store_dwordx4 %0, %1, off " RG_STREAM_STORE_BITS RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
+  else asm volatile("global_store_dwordx4 %0, %1, off" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
 #else
-  if (NT) asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(g), "v"(v));
-  else asm volatile("global_store_dwordx4 %0, %1, off" : : "v"(g), "v"(v));
+  if (NT) asm volatile("global_store_dwordx4 %0, %1, off nt" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
+  else asm volatile("global_store_dwordx4 %0, %1, off" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
 #endif
 }
 template <bool NT> __device__ __forceinline__ void st8_last(char* p, u32x2 v) {
