@@ -15,6 +15,11 @@ import torch
 from .dist_param_locator import DistributedParamLocator
 from .param_storage import ParamStorage
 
+try:        # the compiled module: the registry and the per-step loops over parameters in C++
+    from . import _ranncgrad as _native
+except ImportError:      # not built: the same operations driven from Python over the ctypes binding
+    _native = None
+
 _param_storage = ParamStorage()
 _dist_param_locator = DistributedParamLocator()
 _tracing_state = True
@@ -47,6 +52,8 @@ def clear() -> None:
         _param_storage.undeploy(gid)
     _param_storage = ParamStorage()
     _dist_param_locator.clear()
+    if _native is not None:
+        _native.reset_param_storage()
 
 
 def set_tracing_state(enable: bool) -> None:
@@ -78,6 +85,8 @@ def all_gather(ten: torch.Tensor, buf: torch.Tensor) -> None:
 # -- amp masters (src/main.cpp:191-200)
 def register_amp_master_param(model_param_id: int, param: torch.Tensor) -> None:
     _param_storage.register_amp_master_param(model_param_id, id(param), param)
+    if _native is not None:
+        _native.register_amp_master_param(model_param_id, param)
 
 
 # -- distributed parameters (src/main.cpp:202-245)
@@ -117,18 +126,29 @@ def gather_tensor_zero(ten: torch.Tensor, pid: int) -> torch.Tensor:
     """``src/main.cpp`` ``gather_tensor_zero`` -> ``ParamStorage::gatherTensorZero``
     (``src/comp/ParamStorage.cpp:670-685``): the per-rank pieces of a tensor laid out like the ZeRO
     segments of parameter ``pid``, gathered and viewed in the parameter's shape."""
+    if _native is not None:
+        try:
+            return _native.get_param_storage().gather_tensor_zero(ten, pid)
+        except ValueError:
+            pass                   # deployed through the Python registry (gradient buckets)
     return _param_storage.gather_tensor_zero(ten, pid)
 
 
 def get_param_ranks(pid: int):
-    _param_storage.get_param_tensor(pid)
+    if _native is None or not _native.get_param_storage().has_param(pid):
+        _param_storage.get_param_tensor(pid)
     return {0}
 
 
 class RaNNCModule:
     """The methods of the bound C++ ``RaNNCModule`` (``src/main.cpp:257-450``) that sit on the
-    per-step path.  ``init`` here only registers the parameters of the (whole, unpartitioned)
-    model under one graph id; there is no tracing, profiling or partitioning."""
+    per-step path.  ``init`` only registers the parameters of the (whole, unpartitioned)
+    model under one graph id; there is no tracing, profiling or partitioning.
+
+    The work is done by the class of the same name in the compiled module (``rannc_amd._ranncgrad``: registry and
+    loops over parameters in C++, as in the reference).  Two cases are driven from Python over the ctypes binding
+    instead: ``consolidate_grads`` (the gradient buckets live in ``param_storage.GradConsolidation``) and a
+    package whose compiled module has not been built."""
 
     _next_id = 0
 
@@ -137,13 +157,21 @@ class RaNNCModule:
         self._use_amp_master_params = bool(use_amp_master_params)
         self._allreduce_amp_master_params = bool(allreduce_amp_master_params)
         self._enable_zero = bool(enable_zero)
+        self._ctor_args = (self._use_amp_master_params, self._allreduce_amp_master_params, self._enable_zero,
+                           bool(check_unused_values), bool(offload_params))
         self.graph_id = f"graph_{RaNNCModule._next_id}"
         RaNNCModule._next_id += 1
         self._deployed = False
+        self._n = None            # the compiled class, once ``init`` has chosen it
 
     def init(self, named_params: Dict[str, torch.Tensor], consolidate_grads: bool = False) -> Dict[str, int]:
         """Register ``name -> parameter`` and deploy them; returns ``name -> id``
         (``RaNNCModule::init`` returns the used-parameter ids, ``src/comp/RaNNCModule.cpp:160-501``)."""
+        if _native is not None and not consolidate_grads:
+            self._n = _native.RaNNCModule(*self._ctor_args)
+            ids = self._n.init(dict(named_params), False)
+            self._deployed = True
+            return ids
         ids = {}
         for name, p in named_params.items():
             _param_storage.register_param(id(p), p)
@@ -160,27 +188,38 @@ class RaNNCModule:
 
     def prepare_backward(self) -> None:
         self._check()
-        _param_storage.prepare_backward(self.graph_id)
+        if self._n is None:
+            _param_storage.prepare_backward(self.graph_id)
 
     def allreduce_grads(self) -> None:
         self._check()
+        if self._n is not None:
+            return self._n.allreduce_grads()
         _param_storage.allreduce_param_grads(self.graph_id)
 
     def allreduce_grads_zero(self) -> None:
         self._check()
+        if self._n is not None:
+            return self._n.allreduce_grads_zero()
         self._staging = _param_storage.allreduce_param_grads_zero(self.graph_id)
 
     def clip_grad_norm(self, max_grad_norm: float) -> None:
         self._check()
+        if self._n is not None:
+            return self._n.clip_grad_norm(max_grad_norm)          # narrowed to a C float at the binding
         _param_storage.clip_grad_norm(self.graph_id, float(torch.tensor(max_grad_norm, dtype=torch.float32)),
                                       self._use_amp_master_params)
 
     def calc_grad_norm(self) -> float:
         self._check()
+        if self._n is not None:
+            return self._n.calc_grad_norm()
         return _param_storage.calc_grad_global_l2_norm(self.graph_id, self._use_amp_master_params)
 
     def zero_grad(self) -> None:
         self._check()
+        if self._n is not None:
+            return self._n.zero_grad()
         _param_storage.clear_param_grads(self.graph_id)
 
     def use_amp_master_params(self) -> bool:
@@ -188,22 +227,32 @@ class RaNNCModule:
 
     def align_params(self) -> None:
         self._check()
+        if self._n is not None:
+            return self._n.align_params()
         _param_storage.align_buffer_zero(self.graph_id)
 
     def sync_param_zero(self, grad: bool) -> None:
         self._check()
+        if self._n is not None:
+            return self._n.sync_param_zero(grad)
         _param_storage.bcast_params_zero(self.graph_id, grad)
 
     def set_grad_to_local_param_segment(self) -> None:
         self._check()
+        if self._n is not None:
+            return self._n.set_grad_to_local_param_segment()
         _param_storage.set_grad_to_local_param_segment(self.graph_id)
 
     def get_local_param_range(self, param_id: int) -> Tuple[int, int]:
         self._check()
+        if self._n is not None:
+            return self._n.get_local_param_range(param_id)
         return _param_storage.get_local_param_range(self.graph_id, param_id)
 
     def get_local_param_segment(self, param_id: int) -> torch.Tensor:
         self._check()
+        if self._n is not None:
+            return self._n.get_local_param_segment(param_id)
         return _param_storage.get_local_param_segment(self.graph_id, param_id)
 
     def _owned_tensor(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
@@ -222,12 +271,16 @@ class RaNNCModule:
 
     def get_param(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
         self._check()
+        if self._n is not None:
+            return self._n.get_param(param_id, amp_master_param)
         return self._in_param_shape(self._owned_tensor(param_id, amp_master_param), param_id)
 
     def get_param_grad(self, param_id: int, amp_master_param: bool) -> torch.Tensor:
         """``gatherParamGrad`` (``src/comp/ParamStorage.cpp:1197-1213``): the gradient of the tensor this
         process steps on, zeros when it has none, in the parameter's shape."""
         self._check()
+        if self._n is not None:
+            return self._n.get_param_grad(param_id, amp_master_param)
         owner = self._owned_tensor(param_id, amp_master_param)
         grad = owner.grad if owner.grad is not None else torch.zeros_like(owner)
         return self._in_param_shape(grad, param_id)
@@ -237,6 +290,8 @@ class RaNNCModule:
         root's copy of the parameter (or of its gradient, zeros when it has none) as a fresh tensor on the host;
         ``None`` for a parameter no rank holds (the reference returns an undefined tensor)."""
         self._check()
+        if self._n is not None:
+            return self._n.sync_param_grad(param_id) if grad else self._n.sync_param(param_id)
         if param_id not in _param_storage.params:
             return None
         param = _param_storage.get_param_tensor(param_id)
@@ -254,5 +309,9 @@ class RaNNCModule:
 
     def undeploy(self) -> None:
         if self._deployed:
-            _param_storage.undeploy(self.graph_id)
+            if self._n is not None:
+                self._n.undeploy()
+                self._n = None
+            else:
+                _param_storage.undeploy(self.graph_id)
             self._deployed = False

@@ -26,21 +26,46 @@ HIPCC_FLAGS = [
 
 
 def build_pybind(verbose: bool = True) -> str:
-    """Compile rannc_amd/_ranncgrad (pybind11 entry points over the C ABI; host code only)."""
+    """Compile rannc_amd/_ranncgrad: pybind11 entry points over the C ABI plus the native registry.  Host code only;
+    it sees tensors through PyTorch's C++ headers (as the reference's extension does) and is linked against the
+    libraries of the PyTorch it was built with."""
     import sysconfig
+    from concurrent.futures import ThreadPoolExecutor
 
-    import pybind11
+    import torch
+    from torch.utils import cpp_extension
 
     out = os.path.join(HERE, "_ranncgrad" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
-    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
-           "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"], "-I", os.path.join(ROOT, "include"),
-           os.path.join(HERE, "csrc", "rg_pybind.cpp"), "-o", out + ".tmp",
-           "-L", HERE, "-l:" + LIB_NAME, "-Wl,-rpath,$ORIGIN"]
+    cxx = os.environ.get("CXX", "g++")
+    flags = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-DTORCH_EXTENSION_NAME=_ranncgrad",
+             "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
+    for inc in cpp_extension.include_paths():
+        flags += ["-isystem", inc]
+    flags += ["-I", sysconfig.get_paths()["include"], "-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "csrc")]
+    build_dir = os.path.join(HERE, "build")
+    os.makedirs(build_dir, exist_ok=True)
+    units = ["rg_pybind.cpp", "rg_registry.cpp"]
+
+    def compile_unit(name: str) -> str:
+        obj = os.path.join(build_dir, name + ".o")
+        cmd = [cxx, *flags, "-c", os.path.join(HERE, "csrc", name), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"pybind11 build failed ({proc.returncode}):\n{proc.stdout}")
+        return obj
+
+    with ThreadPoolExecutor(max_workers=len(units)) as pool:
+        objs = list(pool.map(compile_unit, units))
+    torch_lib = cpp_extension.library_paths()[0]
+    cmd = [cxx, "-shared", *objs, "-o", out + ".tmp", "-L", HERE, "-l:" + LIB_NAME, "-L", torch_lib, "-lc10", "-ltorch",
+           "-ltorch_cpu", "-ltorch_python", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
-        raise RuntimeError(f"pybind11 build failed ({proc.returncode}):\n{proc.stdout}")
+        raise RuntimeError(f"pybind11 link failed ({proc.returncode}):\n{proc.stdout}")
     os.replace(out + ".tmp", out)
     return out
 

@@ -3,29 +3,18 @@
 // pybind11 module too (PYBIND11_MODULE(_pyrannc), src/main.cpp:30); like it, this layer only
 // converts arguments (tensor -> pointer, element count, dtype code, current stream) and
 // translates status codes into Python exceptions: std::invalid_argument -> ValueError,
-// std::runtime_error -> RuntimeError.  No torch headers are needed: tensors are inspected
-// through their Python attributes.
-#include <pybind11/pybind11.h>
+// std::runtime_error -> RuntimeError.  This file holds the table classes (Plan, Optim), the
+// plan-free copy and the reference's free functions; rg_registry.cpp adds the native registry
+// (TensorList, GradPlan, ParamStorage, RaNNCModule).
 #include <pybind11/stl.h>
 
-#include <stdexcept>
-#include <string>
 #include <unordered_map>
-#include <vector>
 
-#include "ranncgrad.h"
+#include "rg_bind.h"
 
-namespace py = pybind11;
+using rgbind::check;
 
 namespace {
-
-void check(int rc) {
-  if (rc == RG_OK) return;
-  const std::string msg = rg_last_error();
-  if (rc == RG_EINVAL || rc == RG_EALIGN) throw std::invalid_argument(msg);
-  if (rc == RG_ENOMEM) throw std::bad_alloc();
-  throw std::runtime_error(msg);
-}
 
 int dtype_code(const py::handle& tensor) {
   const std::string name = py::str(tensor.attr("dtype"));
@@ -364,10 +353,6 @@ DistParamRegistry& dist_params() {
   static DistParamRegistry* r = new DistParamRegistry();   // never destroyed: it holds Python objects
   return *r;
 }
-std::unordered_map<long, py::object>& amp_masters() {
-  static auto* m = new std::unordered_map<long, py::object>();
-  return *m;
-}
 
 }  // namespace
 
@@ -412,12 +397,6 @@ PYBIND11_MODULE(_ranncgrad, m) {
       throw std::invalid_argument("all_gather: receive buffer must hold world_size * numel elements");
     copy_cast(buf.attr("view")(-1), ten.attr("contiguous")().attr("view")(-1), 1.0f);
   });
-  m.def("register_amp_master_param", [](long model_param_id, const py::object& param) { amp_masters()[model_param_id] = param; });
-  m.def("get_amp_master_param", [](long model_param_id) {
-    auto it = amp_masters().find(model_param_id);
-    if (it == amp_masters().end()) throw std::invalid_argument("Amp master parameter not found: " + std::to_string(model_param_id));
-    return it->second;
-  });
   m.def("store_dist_param", [](const py::object& param) { return dist_params().store(param); });
   m.def("load_dist_param", [](long pid) { return dist_params().load(pid); });
   m.def("set_dist_param", [](long pid, const py::object& full) { dist_params().set(pid, full); });
@@ -431,8 +410,9 @@ PYBIND11_MODULE(_ranncgrad, m) {
   m.def("dist_param_registered", [](long pid) { return dist_params().registered(pid); });
   m.def("clear", [] {
     dist_params().clear();
-    amp_masters().clear();
+    reset_registry();
   });
+  bind_registry(m);
   py::class_<Plan>(m, "Plan")
       .def(py::init<const py::sequence&, const py::object&, int64_t>(), py::arg("srcs"), py::arg("dsts") = py::none(),
            py::arg("chunk_elems") = 0)
