@@ -175,3 +175,119 @@ def test_dist_param_functions_of_the_compiled_module_match_the_oracle(dtype):
     finally:
         _ranncgrad.remove_dist_param(pid)
     assert not _ranncgrad.dist_param_registered(pid)
+
+
+# ----------------------------------------------------------------------------- the compiled RaNNCModule / ParamStorage
+
+def _named_params(dtypes, seed, dev="cuda:0"):
+    g = torch.Generator().manual_seed(seed)
+    shapes = [(257, 33), (1,), (4099,), (64, 64), (7,)]
+    return {f"layer.{i}.w": torch.nn.Parameter(torch.randn(s, generator=g).to(dt).to(dev))
+            for i, (s, dt) in enumerate(zip(shapes, dtypes))}
+
+
+def test_compiled_module_has_the_reference_methods():
+    """The per-step methods of the reference's bound class (src/main.cpp:333-380)."""
+    for name in ("clip_grad_norm", "calc_grad_norm", "zero_grad", "align_params", "get_local_param_range",
+                 "get_local_param_segment", "use_amp_master_params", "allreduce_grads", "allreduce_grads_zero",
+                 "sync_param_zero", "sync_param", "sync_param_grad", "undeploy"):
+        assert callable(getattr(_ranncgrad.RaNNCModule, name)), name
+    m = _ranncgrad.RaNNCModule(True, False, False, True, False)
+    assert m.use_amp_master_params() is True
+    with pytest.raises(RuntimeError, match="not initialised"):
+        m.clip_grad_norm(1.0)
+    with pytest.raises(ValueError, match="not found"):
+        _ranncgrad.get_param_storage().get_param_tensor(123)
+    with pytest.raises(ValueError, match="not found"):
+        _ranncgrad.get_amp_master_param(123)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtypes", [[torch.float32] * 5, [torch.float16, torch.float32, torch.bfloat16, torch.float16, torch.float32]])
+def test_compiled_module_norm_clip_and_zero_match_the_python_registry(dtypes):
+    """calc_grad_norm / clip_grad_norm / zero_grad of the compiled class against the registry driven from Python
+    over the ctypes binding (same kernels, so the same bits) and against the oracle; one parameter without a
+    gradient; max_grad_norm crossing the binding as a C float."""
+    from rannc_amd.param_storage import ParamStorage
+    named = _named_params(dtypes, seed=31)
+    twins = {n: torch.nn.Parameter(p.detach().clone()) for n, p in named.items()}
+    g = torch.Generator().manual_seed(32)
+    cpu_grads = {}
+    for (n, p), q in zip(named.items(), twins.values()):
+        if n.endswith(".1.w"):
+            continue                                   # no gradient: left out of norm, clip and zero
+        cpu_grads[n] = (torch.randn(p.shape, generator=g) * 0.3).to(p.dtype)
+        p.grad = cpu_grads[n].to(p.device)
+        q.grad = cpu_grads[n].to(q.device)
+    _ranncgrad.reset_param_storage()
+    mod = _ranncgrad.RaNNCModule(False, False, False, True, False)
+    ids = mod.init(named, False)
+    assert list(ids) == sorted(named) and all(ids[n] == id(p) for n, p in named.items())
+    st = ParamStorage()
+    for n, q in twins.items():
+        st.register_param(id(q), q)
+    st.deploy("g", {n: id(q) for n, q in twins.items()})
+    try:
+        want_norm = oracle.grad_global_l2_norm([cpu_grads[n] for n in sorted(cpu_grads)])
+        norm = mod.calc_grad_norm()
+        assert norm == st.calc_grad_global_l2_norm("g", False)
+        assert math.isclose(norm, want_norm, rel_tol=1e-6)
+        mod.clip_grad_norm(0.1)                        # 0.1 is not an fp32 number: narrowed at the binding
+        st.clip_grad_norm("g", float(torch.tensor(0.1, dtype=torch.float32)), False)
+        clipped = [g.clone() for g in (cpu_grads[n] for n in sorted(cpu_grads))]
+        _, coef = oracle.clip_grad_norm(clipped, float(torch.tensor(0.1, dtype=torch.float32)))
+        assert coef is not None
+        for n, p in named.items():
+            if n not in cpu_grads:
+                assert p.grad is None
+                continue
+            assert_bits_equal(p.grad.cpu(), twins[n].grad.cpu(), f"compiled vs ctypes {n}")
+        for got, want in zip((named[n].grad for n in sorted(cpu_grads)), clipped):
+            assert torch.allclose(got.float().cpu(), want.float(), rtol=2e-3 if want.dtype != torch.float32 else 1e-6, atol=0)
+        mod.zero_grad()
+        torch.cuda.synchronize()
+        assert all(p.grad is None or bool((p.grad == 0).all()) for p in named.values())
+    finally:
+        mod.undeploy()
+        st.undeploy("g")
+        _ranncgrad.reset_param_storage()
+
+
+@pytest.mark.gpu
+def test_compiled_module_zero_segments_and_amp_masters():
+    """enable_zero: layouts, local segments and aligned buffers of the compiled class follow the oracle's closed
+    forms at one rank; with amp masters registered the norm is taken over the masters' gradients."""
+    dtypes = [torch.float16] * 5
+    named = _named_params(dtypes, seed=33)
+    before = {n: p.detach().cpu().clone() for n, p in named.items()}
+    _ranncgrad.reset_param_storage()
+    mod = _ranncgrad.RaNNCModule(True, False, True, True, False)
+    ids = mod.init(named, False)
+    try:
+        mod.align_params()
+        torch.cuda.synchronize()
+        masters = {}
+        for n, p in named.items():
+            pid = ids[n]
+            assert_bits_equal(p.detach().cpu(), before[n], "values survive the re-homing")
+            aligned, seg, offs, srcs = _lib.segment_layout(p.numel(), p.element_size(), 1)
+            assert tuple(mod.get_local_param_range(pid)) == (offs[0], offs[0] + srcs[0]) == (0, p.numel())
+            buf = _ranncgrad.get_param_storage().get_buffer(mod.native_graph_id, pid)
+            assert buf.numel() == aligned == oracle.calc_aligned_num_elems(p.numel(), 2, 1)
+            assert bool((buf[p.numel():] == 0).all()) and buf.data_ptr() == p.data_ptr()
+            seg_t = mod.get_local_param_segment(pid)
+            assert seg_t.dim() == 1 and seg_t.data_ptr() == p.data_ptr() and seg_t.requires_grad
+            assert mod.get_local_param_segment(pid) is seg_t or mod.get_local_param_segment(pid).data_ptr() == seg_t.data_ptr()
+            masters[n] = seg_t.detach().clone().float().requires_grad_(True)
+            _ranncgrad.register_amp_master_param(pid, masters[n])
+        g = torch.Generator().manual_seed(34)
+        cpu = {n: torch.randn(m.shape, generator=g) * 0.01 for n, m in masters.items()}
+        for n, m in masters.items():
+            m.grad = cpu[n].to(m.device)
+        want = oracle.grad_global_l2_norm([cpu[n] for n in sorted(cpu)])
+        assert math.isclose(mod.calc_grad_norm(), want, rel_tol=1e-6)
+        with pytest.raises(ValueError, match="not registered"):
+            mod.get_local_param_range(12345)
+    finally:
+        mod.undeploy()
+        _ranncgrad.reset_param_storage()
