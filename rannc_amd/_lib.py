@@ -354,6 +354,11 @@ class OptimTable:
                                   _ptr_array(state1, n), _ptr_array(state2, n), _ptr_array(copies, n),
                                   (C.c_int64 * max(n, 1))(*numels), (C.c_int * max(n, 1))(*grad_dtypes), a_cd))
 
+    @property
+    def handle(self) -> int:
+        """The ``rg_optim*`` as an integer, for another binding of the same library."""
+        return self._handle.value
+
     def update_pointers(self, params=None, grads=None, state1=None, state2=None, copies=None, stream: int = 0) -> None:
         n = self.n
         check(lib.rg_optim_update_pointers(self._handle, _ptr_array(params, n), _ptr_array(grads, n),

@@ -34,6 +34,72 @@ from .. import _lib, _pyrannc
 from ..multi_tensor import TensorPlan
 from ..tensor_coll import _allreduce_min, _allreduce_sum
 
+try:        # the compiled module: the steady state of a training loop walks its parameter lists in C++
+    from .. import _ranncgrad as _native
+except ImportError:
+    _native = None
+
+
+class _StepResult:
+    __slots__ = ("norm", "coef", "overflow", "clipped", "skipped")
+
+    def __init__(self, d) -> None:
+        self.norm, self.coef, self.overflow = d["norm"], d["coef"], d["overflow"]
+        self.clipped, self.skipped = d["clipped"], d["skipped"]
+
+
+class _CompiledStepPlan:
+    """The operations of ``TensorPlan`` that this module uses, over a ``GradPlan`` of the compiled module: a
+    device table that follows the gradients of a fixed list of parameters without a Python loop over them."""
+
+    def __init__(self, grad_plan) -> None:
+        self.gp = grad_plan
+        self.plan = self                       # ``unscale_plan.plan.result_device_ptr()``
+
+    def step_begin(self, inv_scale: float) -> None:
+        self.gp.step_begin(inv_scale)
+
+    def step_finish(self, max_norm: float, flags: int = 0) -> None:
+        self.gp.step_finish(max_norm, flags)
+
+    def step_decide(self, max_norm: float, flags: int = 0) -> None:
+        self.gp.step_decide(max_norm, flags)
+
+    def step_apply_clip(self, max_norm: float, flags: int = 0) -> None:
+        self.gp.step_apply_clip(max_norm, flags)
+
+    def unscale_pack(self, inv_scale: float) -> None:
+        self.gp.unscale_pack(inv_scale)
+
+    def result(self) -> _StepResult:
+        return _StepResult(self.gp.result())
+
+    def result_device_ptr(self) -> int:
+        return self.gp.result_device_ptr()
+
+    def drop_sources(self) -> None:
+        self.gp.drop_sources()
+
+    def is_open(self) -> bool:
+        return self.gp.is_open()
+
+    def close(self) -> None:
+        self.gp.close()
+
+
+class _CompiledLists:
+    """The half parameters, their fp32 masters and the masters' gradient views as lists held by the compiled
+    module, and the table from the half parameters' gradients to those views."""
+
+    def __init__(self, stash: "_AmpStash") -> None:
+        self.n = len(stash.all_fp16_params)
+        self.dtype = stash.all_fp16_params[0].dtype
+        self.half = _native.TensorList(stash.all_fp16_params)
+        self.masters = _native.TensorList(stash.all_fp32_from_fp16_params)
+        self.views = _native.TensorList(stash.master_grad_views)
+        self.grad_plan = _native.GradPlan(self.half, self.views)
+        self.plan = _CompiledStepPlan(self.grad_plan)
+
 
 class _AmpState:
     def __init__(self) -> None:
@@ -64,7 +130,8 @@ class _AmpStash:
         self.pending_model_grads: List[torch.Tensor] = []
         self.decided_max_norm: Optional[float] = None      # clip_grad_norm asked for while the write is pending
         self.fused = False
-        self.last_result = None            # rg_step_result of the last unscale
+        self._last_result = None           # rg_step_result of the last unscale, or the table to read it from
+        self._last_result_plan = None
         # fused mode picks its strategy per step from what the last step did: when it clipped, read pass now and
         # one deferred write pass that applies the coefficient ((2s + d) bytes per element); when it did not, one
         # eager pass that writes while it sums ((s + d)), with an in-place multiply only if this step clips after all
@@ -80,6 +147,24 @@ class _AmpStash:
         # gradients and for adding fresh gradients onto stashed ones (gradient accumulation)
         self.fp32_unscale_plans = None
         self.fp32_accumulate_plans = None
+        self.compiled: Optional[_CompiledLists] = None     # made at the first steady-state exit of scale_loss
+        self.feed = None                   # the GradPlan whose held gradients the pending write / step reads, if any
+
+
+def _get_last_result(stash: _AmpStash):
+    if stash._last_result is None and stash._last_result_plan is not None and stash._last_result_plan.is_open():
+        stash._last_result = stash._last_result_plan.result()
+    return stash._last_result
+
+
+def _set_last_result(stash: _AmpStash, value) -> None:
+    stash._last_result, stash._last_result_plan = value, None
+
+
+#: ``rg_step_result`` of the last unscale.  Under a dynamic loss scale it is read at every ``scale_loss`` exit (the
+#: schedule needs the flag); under a static one nothing on the host depends on it, so it is only fetched - from the
+#: table's result block as the device holds it then - when somebody looks.
+_AmpStash.last_result = property(_get_last_result, _set_last_result)
 
 
 class LossScaler:
@@ -104,7 +189,7 @@ class LossScaler:
         self._has_overflow = False
 
     def unscale(self, stash: _AmpStash, model_grads: List[torch.Tensor], master_grads: List[torch.Tensor],
-                accumulate: bool = False, all_params: bool = False) -> None:
+                accumulate: bool = False, all_params: bool = False, plan=None) -> None:
         """``master_grad = float(model_grad) * (1 / scale)`` for every pair in one launch, with the
         inf/NaN flag and - for free - the gradient norm.  In fused mode only the read pass runs
         here; the values are written by ``finish_unscale``.  ``accumulate`` adds to the master
@@ -118,12 +203,16 @@ class LossScaler:
             stash.unscale_cache = _PlanCache()
         if stash.clip_decided:
             # what the last step decided picks this step's strategy; it is read from the table that took the
-            # decision, before the cache may replace that table by a new one
-            if stash.unscale_plan is not None and stash.unscale_plan.is_open():
+            # decision, before the cache may replace that table by a new one (not at all when the optimizer reads
+            # the model gradients itself: then there is one strategy, and the host does not wait for the device)
+            if (stash.unscale_plan is not None and stash.unscale_plan.is_open()
+                    and not (stash.fused and stash.optimizer_reads_model_grads)):
                 stash.expect_clip = bool(stash.unscale_plan.result().clipped)
             stash.clip_decided = False
         # a new table is tuned on the spot, unless the master gradients hold values that are about to be added to
-        if all_params:
+        if plan is not None:
+            stash.unscale_plan = plan          # a table of the compiled module, already bound to this step's gradients
+        elif all_params:
             stash.unscale_plan = stash.unscale_cache.get_same_shapes("all", model_grads, master_grads, tune_new=not accumulate)
         else:
             stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads, tune_new=not accumulate)
@@ -140,14 +229,18 @@ class LossScaler:
             else:
                 stash.unscale_plan.unscale_pack(inv)
                 stash.sums_cover_all = stash.fused
-        stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
-        if stash.last_result.overflow:
-            self._has_overflow = True
+        if self.dynamic:
+            stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
+            if stash.last_result.overflow:
+                self._has_overflow = True
+        else:
+            stash._last_result, stash._last_result_plan = None, stash.unscale_plan     # a static scale never skips
         if not stash.pending_finish:
             # every kernel that reads the model gradients is queued: let go of them, so that backward
             # finds their memory free again (and, in the steady state, at the same addresses)
             stash.unscale_plan.drop_sources()
             stash.pending_model_grads = []
+            stash.feed = None
 
     def update_scale(self) -> bool:
         """Returns True when the step must be skipped.  Own schedule (see module docstring)."""
@@ -271,6 +364,7 @@ def finish_unscale(optimizer: torch.optim.Optimizer, max_norm: Optional[float] =
         stash.decided_max_norm = None
         stash.unscale_plan.drop_sources()
         stash.pending_model_grads = []
+        stash.feed = None
 
 
 def can_step_from_model_grads(optimizer: torch.optim.Optimizer) -> bool:
@@ -333,13 +427,17 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
             if stash.unscale_plan is not None:
                 stash.unscale_plan.drop_sources()
             stash.pending_model_grads = []
+            stash.feed = None
             return None
         if can_step_from_model_grads(optimizer) and not (args or kwargs):
             # unscale, clip, update and model copy in one kernel: the step reads the still-scaled
             # model gradients and the clip decision from the device
             if stash.decided_max_norm is None:
                 decide_clip(optimizer, 0.0)
-            optimizer.set_grad_sources(stash.pending_masters, stash.pending_model_grads)
+            if stash.feed is not None:
+                optimizer.set_grad_feed(stash.feed, stash.pending_masters)      # read where the compiled table reads
+            else:
+                optimizer.set_grad_sources(stash.pending_masters, stash.pending_model_grads)
             optimizer.grad_scale = stash.pending_inv_scale
             optimizer.gate = stash.unscale_plan.plan.result_device_ptr()
             try:
@@ -351,6 +449,7 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
             stash.decided_max_norm = None
             stash.unscale_plan.drop_sources()
             stash.pending_model_grads = []
+            stash.feed = None
             return ret
         finish_unscale(optimizer)
         ret = old_step(*args, **kwargs)
@@ -393,11 +492,18 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
         stash.master_grad_views = [stash.master_grad_bucket.narrow(0, o, m.numel()).view(m.shape)
                                    for o, m in zip(offs, masters)]
     half_params, masters_all = stash.all_fp16_params, stash.all_fp32_from_fp16_params
-    model_grads_all = [p.grad for p in half_params]
-    n_with_grad = sum(1 for g in model_grads_all if g is not None)
-    n_live = sum(1 for m in masters_all if m.grad is not None)
     scaler.clear_overflow_state()
-    if n_with_grad == len(half_params) and n_live == 0 and half_params:
+    dropped_half_grads = False
+    if _native is not None and half_params and _compiled_steady_exit(stash, scaler):
+        dropped_half_grads = True
+        model_grads_all, n_with_grad, n_live = [], -1, 0
+    else:
+        model_grads_all = [p.grad for p in half_params]
+        n_with_grad = sum(1 for g in model_grads_all if g is not None)
+        n_live = sum(1 for m in masters_all if m.grad is not None)
+    if dropped_half_grads:
+        pass
+    elif n_with_grad == len(half_params) and n_live == 0 and half_params:
         # The steady state of a training loop: every half parameter has a fresh gradient and no master gradient
         # is alive (zero_grad dropped them).  Nothing is classified or sorted; the table keeps its shape.
         views = stash.master_grad_views
@@ -450,18 +556,44 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
         if fresh32:
             plan = stash.fp32_unscale_plans.get(fresh32, fresh32)
             plan.unscale_pack(inv)
-            if plan.result().overflow:
+            if scaler.dynamic and plan.result().overflow:       # a static scale never skips: nothing waits for the flag
                 scaler._has_overflow = True
         if new32:
             plan = stash.fp32_accumulate_plans.get(new32, old32)
             plan.unscale_accumulate(inv)
-            if plan.result().overflow:
+            if scaler.dynamic and plan.result().overflow:       # a static scale never skips: nothing waits for the flag
                 scaler._has_overflow = True
     should_skip = scaler.update_scale()
     if should_skip:
         stash.skip_next_step = True
-    for p in stash.all_fp16_params:       # Apex O2 drops the half grads once they are unscaled
-        p.grad = None
+    if not dropped_half_grads:
+        for p in stash.all_fp16_params:       # Apex O2 drops the half grads once they are unscaled
+            p.grad = None
+
+
+def _compiled_steady_exit(stash: _AmpStash, scaler: LossScaler) -> bool:
+    """The steady state of a training loop - every half parameter has a fresh, contiguous gradient of its own dtype
+    and no master gradient is alive - handled without a Python loop over the parameters: the compiled module
+    counts the gradients, hangs the bucket views on the masters, re-points its table at the new gradients,
+    and drops the half gradients once the kernels that read them are queued.  Returns False, having changed
+    nothing, when the step is not of that kind (the general path then runs)."""
+    lists = stash.compiled
+    if lists is None:
+        if any(p.dtype != stash.all_fp16_params[0].dtype for p in stash.all_fp16_params):
+            return False
+        lists = stash.compiled = _CompiledLists(stash)
+    if lists.half.steady_grads(lists.dtype) != lists.n or lists.masters.count_grads() != 0:
+        return False
+    lists.masters.set_grads(lists.views)
+    if lists.grad_plan.bind() != lists.n:
+        raise RuntimeError("the gradients of the half parameters changed while they were being bound")
+    if lists.grad_plan.rebuilt():
+        lists.grad_plan.tune()               # the views hold nothing yet: measure the write order on them
+    stash.pending_masters, stash.pending_model_grads = stash.all_fp32_from_fp16_params, None
+    stash.feed = lists.grad_plan
+    scaler.unscale(stash, None, None, accumulate=False, plan=lists.plan)
+    lists.half.clear_grads()                 # Apex O2 drops the half grads once they are unscaled
+    return True
 
 
 # --------------------------------------------------------------------------- reference API
@@ -552,6 +684,7 @@ def unset_master_grads(optimizer):
         stash.decided_max_norm = None
         stash.unscale_plan.drop_sources()
         stash.pending_model_grads = []
+        stash.feed = None
     for group in optimizer.param_groups:
         for p in group["params"]:
             p.grad = None

@@ -168,6 +168,7 @@ class GradPlan {
     held_.clear();
   }
   int64_t num_chunks() { return rg_plan_num_chunks(plan_.get()); }
+  uintptr_t handle() { return reinterpret_cast<uintptr_t>(plan_.get()); }   // the rg_plan*, for telling tables apart
 
  private:
   std::shared_ptr<TensorList> owners_, dsts_;
@@ -658,7 +659,8 @@ void bind_registry(py::module_& m) {
       .def("result_device_ptr", &GradPlan::result_device_ptr)
       .def("is_open", &GradPlan::is_open)
       .def("close", &GradPlan::close)
-      .def_property_readonly("num_chunks", &GradPlan::num_chunks);
+      .def_property_readonly("num_chunks", &GradPlan::num_chunks)
+      .def_property_readonly("handle", &GradPlan::handle);
 
   py::class_<ParamStorage, std::shared_ptr<ParamStorage>>(m, "ParamStorage")
       .def(py::init<>())

@@ -18,6 +18,11 @@ import torch
 from . import _lib
 from .multi_tensor import dtype_code, stream_handle
 
+try:        # the compiled module: lists of parameters walked in C++
+    from . import _ranncgrad as _native
+except ImportError:
+    _native = None
+
 
 _data_ptr = torch.Tensor.data_ptr
 _is_contiguous = torch.Tensor.is_contiguous
@@ -27,7 +32,7 @@ class _Steady:
     """What a group's last full step established, for the steps after it: as long as the same parameters all
     have contiguous gradients of the same dtype, a step is one pointer comparison per gradient and one launch."""
     __slots__ = ("params_obj", "n", "param_ids", "table", "key", "grad_ptrs", "grad_dtype", "steps_buf", "count", "device",
-                 "param_ptr_ends")
+                 "param_ptr_ends", "fed_by")
 
 
 class _FusedBase(torch.optim.Optimizer):
@@ -46,6 +51,10 @@ class _FusedBase(torch.optim.Optimizer):
         #: every gradient is multiplied by this first
         self.grad_scale: float = 1.0
         self._grad_sources: Dict[int, torch.Tensor] = {}
+        self._feed = None                          # see set_grad_feed
+        self._feed_params: List[torch.Tensor] = []
+        self._feed_offsets: Optional[Dict[int, int]] = None
+        self._native_lists: Dict[int, Tuple] = {}  # group index -> (its params list, its length, compiled TensorList)
 
     #: the step can read gradients from tensors other than ``param.grad`` (see ``set_grad_sources``)
     reads_grad_sources = True
@@ -56,6 +65,33 @@ class _FusedBase(torch.optim.Optimizer):
         with ``grad_scale`` and ``gate`` this folds unscale and clip into the step.  Empty lists
         switch it off."""
         self._grad_sources = {id(p): g for p, g in zip(params, grads) if g is not None}
+        self._feed, self._feed_params, self._feed_offsets = None, [], None
+
+    def set_grad_feed(self, feed, params) -> None:
+        """``set_grad_sources`` for gradients that a table of the compiled module (a ``GradPlan``) holds:
+        ``params[i]`` reads the plan's i-th gradient.  A group whose parameters are a run of ``params`` and whose
+        last step left a steady-state record gets the new addresses pushed into its table by the compiled module -
+        no Python loop over the parameters; anything else falls back to the tensors themselves."""
+        self._grad_sources = {}
+        self._feed, self._feed_params = feed, params
+        offsets: Optional[Dict[int, int]] = {}
+        off = 0
+        for gi, group in enumerate(self.param_groups):
+            ps = group["params"]
+            n = len(ps)
+            if n == 0:
+                continue
+            if off + n > len(params) or ps[0] is not params[off] or ps[-1] is not params[off + n - 1]:
+                offsets = None
+                break
+            offsets[gi] = off
+            off += n
+        self._feed_offsets = offsets
+
+    def _sources_from_feed(self) -> None:
+        """The fed gradients as tensors, for the paths that look at every parameter."""
+        if self._feed is not None and not self._grad_sources:
+            self._grad_sources = {id(p): g for p, g in zip(self._feed_params, self._feed.sources()) if g is not None}
 
     def load_state_dict(self, state_dict) -> None:
         super().load_state_dict(state_dict)
@@ -77,6 +113,22 @@ class _FusedBase(torch.optim.Optimizer):
         params = group["params"]
         if st is None or st.params_obj is not params or len(params) != st.n:
             return None
+        if self._feed is not None and not self._grad_sources:
+            off = self._feed_offsets.get(gi) if self._feed_offsets is not None else None
+            if (off is not None and self._feed.held() >= off + st.n and dtype_code(st.grad_dtype) == self._feed.source_dtype()
+                    and (params[0].data_ptr(), params[-1].data_ptr()) == st.param_ptr_ends):
+                if st.fed_by is not self._feed:
+                    self._feed.forget_optim(st.table.handle)      # whatever an earlier table at this address was told
+                    st.fed_by = self._feed
+                if self._feed.push_sources_to_optim(st.table.handle, off, st.n) or st.grad_ptrs is not None:
+                    # the table was re-pointed behind the back of the records kept here: they no longer say where it
+                    # points, so that a later step through the general path pushes every address again
+                    st.grad_ptrs = None
+                    hit = self._tables.get(st.key)
+                    if hit is not None and hit[0] is st.table:
+                        self._tables[st.key] = (hit[0], None, hit[2])
+                return st, None
+            self._sources_from_feed()
         if self._grad_sources:
             grads = list(map(self._grad_sources.get, st.param_ids))
         else:
@@ -101,7 +153,7 @@ class _FusedBase(torch.optim.Optimizer):
             # the full path's record of what the table points at must not outlive this re-pointing: a later
             # full step with the old addresses would otherwise find them "unchanged" and skip the update
             hit = self._tables.get(st.key)
-            if hit is not None and hit[0] is st.table:
+            if hit is not None and hit[0] is st.table and hit[1] is not None:
                 self._tables[st.key] = (hit[0], (hit[1][0], tuple(ptrs)) + tuple(hit[1][2:]), hit[2])
         return st, grads
 
@@ -114,6 +166,7 @@ class _FusedBase(torch.optim.Optimizer):
         st.key = table.cache_key
         st.param_ptr_ends = (params[0].data_ptr(), params[-1].data_ptr())
         st.grad_ptrs = [g.data_ptr() for g in grads]
+        st.fed_by = None
         st.grad_dtype = grads[0].dtype
         st.device = params[0].device
         st.count = count
@@ -130,11 +183,20 @@ class _FusedBase(torch.optim.Optimizer):
         """``torch.optim.Optimizer.zero_grad`` without its per-parameter bookkeeping."""
         if not set_to_none:
             return super().zero_grad(set_to_none=False)
-        for group in self.param_groups:
-            for p in group["params"]:
-                p.grad = None
+        for gi, group in enumerate(self.param_groups):
+            params = group["params"]
+            if _native is None:
+                for p in params:
+                    p.grad = None
+                continue
+            known = self._native_lists.get(gi)
+            if known is None or known[0] is not params or known[1] != len(params):
+                known = self._native_lists[gi] = (params, len(params), _native.TensorList(params))
+            known[2].clear_grads()
 
     def _grad_of(self, p: torch.Tensor) -> Optional[torch.Tensor]:
+        if self._feed is not None:
+            self._sources_from_feed()
         return self._grad_sources.get(id(p), p.grad) if self._grad_sources else p.grad
 
     # -- model copies (amp): written by the step kernel instead of a separate copy pass

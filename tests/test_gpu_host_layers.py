@@ -393,10 +393,12 @@ def test_amp_keeps_one_device_table_across_steps(fused):
             if step == 2:       # make backward's next allocation land elsewhere: the table must follow, not be rebuilt
                 hold = [torch.empty_like(p.grad) for p in opt._amp_stash.all_fp16_params]
         stash = opt._amp_stash
-        handles.add(stash.unscale_plan.plan._handle.value)
+        plan = stash.unscale_plan                  # a table of the compiled module, or a TensorPlan over ctypes
+        handles.add(plan.gp.handle if hasattr(plan, "gp") else plan.plan._handle.value)
         rm.clip_grad_norm(1.0)
         opt.step()
-        assert all(s is None for s in stash.unscale_plan._srcs) and stash.pending_model_grads == []
+        held = plan.gp.held() if hasattr(plan, "gp") else sum(s is not None for s in plan._srcs)
+        assert held == 0 and stash.pending_model_grads == []
         opt.zero_grad()
     assert len(handles) == 1
     del hold
