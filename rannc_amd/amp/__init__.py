@@ -582,11 +582,8 @@ def _compiled_steady_exit(stash: _AmpStash, scaler: LossScaler) -> bool:
         if any(p.dtype != stash.all_fp16_params[0].dtype for p in stash.all_fp16_params):
             return False
         lists = stash.compiled = _CompiledLists(stash)
-    if lists.half.steady_grads(lists.dtype) != lists.n or lists.masters.count_grads() != 0:
+    if lists.grad_plan.bind_steady(lists.masters, lists.dtype) != lists.n:
         return False
-    lists.masters.set_grads(lists.views)
-    if lists.grad_plan.bind() != lists.n:
-        raise RuntimeError("the gradients of the half parameters changed while they were being bound")
     if lists.grad_plan.rebuilt():
         lists.grad_plan.tune()               # the views hold nothing yet: measure the write order on them
     stash.pending_masters, stash.pending_model_grads = stash.all_fp32_from_fp16_params, None

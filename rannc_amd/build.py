@@ -37,7 +37,9 @@ def build_pybind(verbose: bool = True) -> str:
 
     out = os.path.join(HERE, "_ranncgrad" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
     cxx = os.environ.get("CXX", "g++")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     flags = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-DTORCH_EXTENSION_NAME=_ranncgrad",
+             "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM", "-isystem", os.path.join(rocm, "include"),      # c10/hip/HIPStream.h
              "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
     for inc in cpp_extension.include_paths():
         flags += ["-isystem", inc]
@@ -59,7 +61,7 @@ def build_pybind(verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=len(units)) as pool:
         objs = list(pool.map(compile_unit, units))
     torch_lib = cpp_extension.library_paths()[0]
-    cmd = [cxx, "-shared", *objs, "-o", out + ".tmp", "-L", HERE, "-l:" + LIB_NAME, "-L", torch_lib, "-lc10", "-ltorch",
+    cmd = [cxx, "-shared", *objs, "-o", out + ".tmp", "-L", HERE, "-l:" + LIB_NAME, "-L", torch_lib, "-lc10", "-lc10_hip", "-ltorch",
            "-ltorch_cpu", "-ltorch_python", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -4,6 +4,7 @@
 // only when the pairs change shape and re-pointed when they only move.
 #pragma once
 
+#include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
 #include <stdexcept>
@@ -36,10 +37,10 @@ inline int dtype_code(const at::Tensor& t) {
   }
 }
 
-// hipStream_t of PyTorch's current stream on `device`, asked of PyTorch itself.
+// hipStream_t of PyTorch's current stream on `device`, asked of PyTorch's own stream registry (what
+// torch.cuda.current_stream(device).cuda_stream reads, without the trip through Python).
 inline void* current_stream(int device) {
-  static py::object* fn = new py::object(py::module_::import("torch").attr("cuda").attr("current_stream"));
-  return reinterpret_cast<void*>((*fn)(device).attr("cuda_stream").cast<uintptr_t>());
+  return reinterpret_cast<void*>(c10::hip::getCurrentHIPStream((c10::DeviceIndex)device).stream());
 }
 
 inline void require_gpu_contiguous(const at::Tensor& t, const char* what, size_t i) {

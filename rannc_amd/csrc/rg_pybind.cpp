@@ -47,11 +47,7 @@ Ref tensor_ref(const py::handle& t, const char* what, size_t i) {
   return r;
 }
 
-void* current_stream(int device) {
-  py::object torch = py::module_::import("torch");
-  py::object s = torch.attr("cuda").attr("current_stream")(device);
-  return reinterpret_cast<void*>(s.attr("cuda_stream").cast<uintptr_t>());
-}
+using rgbind::current_stream;
 
 struct Tables {
   std::vector<const void*> src;

@@ -103,6 +103,21 @@ class GradPlan {
     return bound_;
   }
   bool rebuilt() const { return rebuilt_; }
+  // bind() for the steady state of a mixed-precision loop, in one walk: every owner (half parameter) has a usable
+  // gradient - on the GPU, contiguous, of `dtype`, of its size - and no master has one yet; then each master's
+  // gradient becomes its destination view and the table is bound.  -1, with nothing changed, otherwise.
+  int bind_steady(TensorList& masters, at::ScalarType dtype) {
+    if (!dsts_ || masters.size() != owners_->size()) throw std::invalid_argument("bind_steady: one master and one view per owner");
+    const auto& owners = owners_->tensors();
+    const auto& ms = masters.tensors();
+    for (size_t i = 0; i < owners.size(); ++i) {
+      const at::Tensor& g = owners[i].grad();
+      if (!g.defined() || !g.is_cuda() || !g.is_contiguous() || g.scalar_type() != dtype || g.numel() != owners[i].numel()) return -1;
+      if (ms[i].grad().defined()) return -1;
+    }
+    masters.set_grads(*dsts_);
+    return bind();
+  }
   // The gradient addresses the table reads, handed to an optimizer table (an rg_optim made by any binding of the
   // library) whose rows [0, count) are the owners [offset, offset + count) of this plan: one stream-ordered
   // upload, and none when that table already points there.
@@ -636,6 +651,9 @@ void bind_registry(py::module_& m) {
       .def(py::init<std::shared_ptr<TensorList>, std::shared_ptr<TensorList>>(), py::arg("owners"), py::arg("dsts") = nullptr)
       .def("bind", &GradPlan::bind)
       .def("rebuilt", &GradPlan::rebuilt)
+      .def("bind_steady", [](GradPlan& p, TensorList& masters, const py::object& dtype) {
+             return p.bind_steady(masters, torch::python::detail::py_object_to_dtype(dtype));
+           })
       .def("push_sources_to_optim", &GradPlan::push_sources_to_optim, py::arg("optim_handle"), py::arg("offset"), py::arg("count"))
       .def("forget_optim", &GradPlan::forget_optim)
       .def("held", &GradPlan::held)
