@@ -405,11 +405,12 @@ def run_ceilings(steps: int, warmup: int, nbytes: int = 1 << 30) -> list:
     from rannc_amd import _lib
     from rannc_amd.multi_tensor import stream_handle
     dev = torch.device("cuda", 0)
-    arrays = [torch.empty(nbytes // 4, dtype=torch.float32, device=dev).fill_(1.0) for _ in range(4)]
+    arrays = [torch.empty(nbytes // 4, dtype=torch.float32, device=dev).fill_(1.0) for _ in range(5)]
     ptrs = [a.data_ptr() for a in arrays]
     out = []
     for name, kind, moved in (("read", 0, 1.0), ("fill", 1, 1.0), ("copy_f32", 2, 2.0), ("copy_f32_nt", 5, 2.0),
-                              ("widen_bf16_f32", 3, 1.5), ("adam_streams", 4, 7.0)):
+                              ("widen_bf16_f32", 3, 1.5), ("adam_streams", 4, 7.0), ("adam_streams_bf16_copy", 6, 7.5),
+                              ("adam_streams_bf16_copy_step_shape", 7, 7.5)):
         def fn():
             _lib.ceiling_kernel(kind, ptrs, nbytes, 0, stream_handle(dev))
         wall, dev_s = timed(fn, steps, warmup, 20)
@@ -417,8 +418,9 @@ def run_ceilings(steps: int, warmup: int, nbytes: int = 1 << 30) -> list:
         out.append({"workload": "flat_1GiB", "op": "ceiling_" + name, "ms_per_step": round(dev_s * 1e3, 4),
                     "algorithmic_bytes_per_step": b, "GB/s": round(b / dev_s / 1e9, 1),
                     "pct_of_hbm_peak": round(100.0 * b / dev_s / 1e9 / HBM_PEAK_GBPS, 2), "steps": steps})
-        if name == "adam_streams":
-            arrays[0].fill_(1.0)
+        if name.startswith("adam_streams"):
+            for a in arrays[:4]:
+                a.fill_(1.0)
     del arrays
     torch.cuda.empty_cache()
     return out

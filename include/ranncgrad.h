@@ -362,7 +362,9 @@ int rg_plan_read_timing(rg_plan* plan, int slot, float ms[4]);
  *   kind 2  fp32 copy * 1.5       arrays: src[nbytes], dst[nbytes]
  *   kind 3  bf16 -> fp32 * 0.5    arrays: src[nbytes / 2], dst[nbytes]
  *   kind 4  Adam's streams        arrays: p, g, m, v [nbytes each]; p, m, v rewritten in place
- *   kind 5  kind 2 with the compiler's plain nontemporal stores instead of the write passes' cache policy */
+ *   kind 5  kind 2 with the compiler's plain nontemporal stores instead of the write passes' cache policy
+ *   kind 6  kind 4 + a bf16 copy  arrays: p, g, m, v [nbytes each], copy[nbytes / 2] written (the step under mixed precision)
+ *   kind 7  kind 6 in the optimizer step's launch shape (256 threads over 4096 elements, four vectors per array in flight) */
 int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, int64_t nbytes, int device, void* stream);
 
 #ifdef __cplusplus

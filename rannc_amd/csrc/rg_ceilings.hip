@@ -42,8 +42,9 @@ __global__ __launch_bounds__(256) void ceiling_read_kernel(const char* src, int6
 // wider side (one 4 KiB page of fp32 per block).
 // kind 1: fill (write only)   2: fp32 copy   3: bf16 -> fp32 widening copy   4: four fp32 streams
 // read, three of them written in place (Adam's pattern)   5: fp32 copy with plain `nt` stores
+// 6: kind 4 plus the bf16 model copy as an eighth stream (the optimizer step under mixed precision)
 template <int KIND>
-__global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, char* a2, char* a3, int64_t nvec) {
+__global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, char* a2, char* a3, char* a4, int64_t nvec) {
   const int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x;
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, 
       x.z = __uint_as_float(h.y << 16);
       x.w = __uint_as_float(h.y & 0xffff0000u);
       st16_stream(a1 + i * 16, as_u32x4(x * 0.5f));
-    } else {
+    } else {   // 4 and 6
       const f32x4 p = as_f32x4(ld16_a4<true>(a0 + i * 16));
       const f32x4 g = as_f32x4(ld16_a4<true>(a1 + i * 16));
       const f32x4 m = as_f32x4(ld16_a4<true>(a2 + i * 16));
@@ -77,7 +78,40 @@ __global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, 
       st16<true>(a0 + i * 16, as_u32x4(p2));
       st16<true>(a2 + i * 16, as_u32x4(m2));
       st16<true>(a3 + i * 16, as_u32x4(v2));
+      if constexpr (KIND == 6) {
+        const u32x2 h = {f32x2_to_bf16x2_bits(p2.x, p2.y), f32x2_to_bf16x2_bits(p2.z, p2.w)};
+        st8<true>(a4 + i * 8, h);
+      }
     }
+  }
+}
+
+// Kind 7: the streams of kind 6 in the optimizer step's own launch shape - 256 threads over 4096 elements, the
+// four vectors of every array in flight together - still over flat arrays.
+__global__ __launch_bounds__(256) void ceiling_adam_shape_kernel(char* a0, char* a1, char* a2, char* a3, char* a4, int64_t nvec) {
+  const int64_t base = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+  u32x4 p[4], g[4], m[4], v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    int64_t i = base + u * 256;
+    if (i >= nvec) i = nvec - 1;
+    p[u] = ld16_a4<true>(a0 + i * 16);
+    g[u] = ld16_a4<true>(a1 + i * 16);
+    m[u] = ld16_a4<true>(a2 + i * 16);
+    v[u] = ld16_a4<true>(a3 + i * 16);
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int64_t i = base + u * 256;
+    if (i >= nvec) return;
+    const f32x4 m2 = as_f32x4(m[u]) + 0.1f * (as_f32x4(g[u]) - as_f32x4(m[u]));
+    const f32x4 v2 = as_f32x4(v[u]) * 0.999f + 0.001f * as_f32x4(g[u]) * as_f32x4(g[u]);
+    const f32x4 p2 = as_f32x4(p[u]) - 0.001f * m2;
+    st16<true>(a0 + i * 16, as_u32x4(p2));
+    st16<true>(a2 + i * 16, as_u32x4(m2));
+    st16<true>(a3 + i * 16, as_u32x4(v2));
+    const u32x2 h = {f32x2_to_bf16x2_bits(p2.x, p2.y), f32x2_to_bf16x2_bits(p2.z, p2.w)};
+    st8<true>(a4 + i * 8, h);
   }
 }
 
@@ -87,8 +121,8 @@ __global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, 
 using namespace rg;
 
 RG_API int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, int64_t nbytes, int device, void* stream) {
-  static const int need[6] = {2, 1, 2, 2, 4, 2};
-  if (kind < 0 || kind > 5 || arrays_dev == nullptr || n_arrays < need[kind] || nbytes < 16 || nbytes % 16 != 0) {
+  static const int need[8] = {2, 1, 2, 2, 4, 2, 5, 5};
+  if (kind < 0 || kind > 7 || arrays_dev == nullptr || n_arrays < need[kind] || nbytes < 16 || nbytes % 16 != 0) {
     set_error("rg_ceiling_kernel: bad arguments (kind %d, %d arrays, %lld bytes)", kind, n_arrays, (long long)nbytes);
     return RG_EINVAL;
   }
@@ -99,8 +133,8 @@ RG_API int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, in
     }
   }
   const int64_t nvec = nbytes / 16;   // 16-byte vectors of the widest stream
-  char* a[4] = {nullptr, nullptr, nullptr, nullptr};
-  for (int i = 0; i < need[kind] && i < 4; ++i) a[i] = static_cast<char*>(arrays_dev[i]);
+  char* a[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  for (int i = 0; i < need[kind] && i < 5; ++i) a[i] = static_cast<char*>(arrays_dev[i]);
   DeviceGuard guard(device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (kind == 0) {
@@ -114,6 +148,16 @@ RG_API int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, in
     RG_HIP(hipGetLastError());
     return RG_OK;
   }
+  if (kind == 7) {
+    const int64_t blocks = (nvec + 1023) / 1024;
+    if (blocks > 0x7fffffffLL) {
+      set_error("rg_ceiling_kernel: too large for one launch");
+      return RG_EINVAL;
+    }
+    hipLaunchKernelGGL(ceiling_adam_shape_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a[0], a[1], a[2], a[3], a[4], nvec);
+    RG_HIP(hipGetLastError());
+    return RG_OK;
+  }
   const int64_t blocks = (nvec + 255) / 256;
   if (blocks > 0x7fffffffLL) {
     set_error("rg_ceiling_kernel: too large for one launch");
@@ -121,11 +165,12 @@ RG_API int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, in
   }
   const dim3 grid((unsigned)blocks), block(128);
   switch (kind) {
-    case 1: hipLaunchKernelGGL(ceiling_write_kernel<1>, grid, block, 0, s, a[0], a[1], a[2], a[3], nvec); break;
-    case 2: hipLaunchKernelGGL(ceiling_write_kernel<2>, grid, block, 0, s, a[0], a[1], a[2], a[3], nvec); break;
-    case 3: hipLaunchKernelGGL(ceiling_write_kernel<3>, grid, block, 0, s, a[0], a[1], a[2], a[3], nvec); break;
-    case 4: hipLaunchKernelGGL(ceiling_write_kernel<4>, grid, block, 0, s, a[0], a[1], a[2], a[3], nvec); break;
-    default: hipLaunchKernelGGL(ceiling_write_kernel<5>, grid, block, 0, s, a[0], a[1], a[2], a[3], nvec); break;
+    case 1: hipLaunchKernelGGL(ceiling_write_kernel<1>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
+    case 2: hipLaunchKernelGGL(ceiling_write_kernel<2>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
+    case 3: hipLaunchKernelGGL(ceiling_write_kernel<3>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
+    case 4: hipLaunchKernelGGL(ceiling_write_kernel<4>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
+    case 6: hipLaunchKernelGGL(ceiling_write_kernel<6>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
+    default: hipLaunchKernelGGL(ceiling_write_kernel<5>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
   }
   RG_HIP(hipGetLastError());
   return RG_OK;
