@@ -336,6 +336,44 @@ typedef struct rg_sgd_args {
 } rg_sgd_args;
 int rg_sgd_step(rg_optim* opt, const rg_sgd_args* args, void* stream);
 
+/* ---------------------------------------------------------------- loss scale on the device */
+
+/* The dynamic loss-scale schedule as a one-thread kernel, so that a mixed-precision step needs no host read:
+ * the reference reads the overflow flag back every step and updates the scale on the host
+ * (pyrannc/amp/__init__.py:44-65 around Apex's LossScaler.update_scale; Apex is pinned at
+ * docker/ubuntu/runtime/Dockerfile:13).  An rg_scaler_state is 32 bytes of device memory owned by the caller.
+ * rg_scaler_update applies, to the `overflow` flag of a plan's result block:
+ *   overflow and RG_SCALER_DYNAMIC:  loss_scale /= 2, floored at min_loss_scale when that is > 0, then truncated
+ *                                    to an integer under RG_SCALER_TRUNCATE (what the reference's all-reduce of
+ *                                    int(loss_scale) leaves, :57-61); unskipped = 0; skipped_steps += 1
+ *   otherwise:                       unskipped += 1
+ *   unskipped == scale_window and RG_SCALER_DYNAMIC:  loss_scale = min(max_loss_scale, loss_scale * scale_factor);
+ *                                    unskipped = 0
+ * and stores inv_scale = float(1 / double(loss_scale)).  A static scale (no RG_SCALER_DYNAMIC) only counts.
+ * rg_step_begin_scaled is rg_step_begin with inv_scale read from device memory (normally &state->inv_scale) by
+ * the kernels; rg_step_finish / rg_step_decide follow it as they follow rg_step_begin.
+ * rg_optim_set_grad_scale_source makes every later step of an optimizer table multiply the gradients by the float
+ * at `grad_scale_dev` instead of args->grad_scale (NULL: back to the argument).
+ * Order on one stream: rg_step_begin_scaled -> rg_step_decide / rg_step_finish -> [optimizer step, gated] ->
+ * rg_scaler_update; the next rg_step_begin_scaled then reads the new inv_scale.  All of it can be recorded in
+ * a HIP graph. */
+typedef struct rg_scaler_state {
+  float loss_scale;
+  float inv_scale;        /* 1 / loss_scale, what the next unscale multiplies by */
+  int32_t unskipped;      /* clean steps since the scale last changed */
+  int32_t skipped_steps;  /* steps skipped so far */
+  float min_loss_scale;   /* 0: no floor */
+  float max_loss_scale;
+  int32_t scale_window;
+  float scale_factor;
+} rg_scaler_state;
+enum { RG_SCALER_DYNAMIC = 1, RG_SCALER_TRUNCATE = 2 };
+/* Writes *init_host (inv_scale recomputed) into state_dev with a kernel on `stream`. */
+int rg_scaler_init(rg_scaler_state* state_dev, const rg_scaler_state* init_host, int device, void* stream);
+int rg_scaler_update(rg_scaler_state* state_dev, const rg_step_result* result_dev, int flags, int device, void* stream);
+int rg_step_begin_scaled(rg_plan* plan, const float* inv_scale_dev, void* stream);
+int rg_optim_set_grad_scale_source(rg_optim* opt, const float* grad_scale_dev);
+
 /* ---------------------------------------------------------------- per-kernel timing */
 
 /* Optional profiling aid (no counterpart in the reference, which times with its own

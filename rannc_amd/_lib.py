@@ -60,6 +60,10 @@ SIGNATURES = {
     "rg_plan_set_write_order": (_i, [_vp, _i]),
     "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
     "rg_step_begin": (_i, [_vp, _f, _vp]),
+    "rg_step_begin_scaled": (_i, [_vp, _vp, _vp]),
+    "rg_scaler_init": (_i, [_vp, _vp, _i, _vp]),
+    "rg_scaler_update": (_i, [_vp, _vp, _i, _i, _vp]),
+    "rg_optim_set_grad_scale_source": (_i, [_vp, _vp]),
     "rg_step_finish": (_i, [_vp, _f, _i, _vp]),
     "rg_step_decide": (_i, [_vp, _f, _i, _vp]),
     "rg_unscale_pack": (_i, [_vp, _f, _vp]),
@@ -233,6 +237,10 @@ class Plan:
     def step_begin(self, inv_scale: float, stream: int = 0) -> None:
         check(lib.rg_step_begin(self._handle, inv_scale, _vp(stream)))
 
+    def step_begin_scaled(self, inv_scale_ptr: int, stream: int = 0) -> None:
+        """``step_begin`` with ``inv_scale`` read by the kernels from device memory (a scaler state's ``inv_scale``)."""
+        check(lib.rg_step_begin_scaled(self._handle, _vp(inv_scale_ptr), _vp(stream)))
+
     def step_finish(self, max_norm: float, flags: int = RG_STEP_DEFAULT, stream: int = 0) -> None:
         check(lib.rg_step_finish(self._handle, max_norm, flags, _vp(stream)))
 
@@ -329,6 +337,29 @@ def _ptr_array(ptrs: Optional[Sequence[Optional[int]]], n: int):
     return (C.c_void_p * max(n, 1))(*[p if p else None for p in ptrs])
 
 
+class ScalerState(C.Structure):
+    """``rg_scaler_state``: the loss scale and its schedule as they sit in 32 bytes of device memory."""
+    _fields_ = [("loss_scale", C.c_float), ("inv_scale", C.c_float), ("unskipped", C.c_int32), ("skipped_steps", C.c_int32),
+                ("min_loss_scale", C.c_float), ("max_loss_scale", C.c_float), ("scale_window", C.c_int32),
+                ("scale_factor", C.c_float)]
+
+
+SCALER_STATE_BYTES = C.sizeof(ScalerState)
+SCALER_INV_SCALE_OFFSET = ScalerState.inv_scale.offset
+RG_SCALER_DYNAMIC, RG_SCALER_TRUNCATE = 1, 2
+
+
+def scaler_init(state_ptr: int, loss_scale: float, min_loss_scale: float, max_loss_scale: float, scale_window: int,
+                scale_factor: float, device: int, stream: int = 0) -> None:
+    init = ScalerState(loss_scale, 0.0, 0, 0, min_loss_scale or 0.0, max_loss_scale, scale_window, scale_factor)
+    check(lib.rg_scaler_init(_vp(state_ptr), C.byref(init), device, _vp(stream)))
+
+
+def scaler_update(state_ptr: int, result_ptr: int, flags: int, device: int, stream: int = 0) -> None:
+    """One thread applies the loss-scale schedule to the overflow flag of a plan's result block."""
+    check(lib.rg_scaler_update(_vp(state_ptr), _vp(result_ptr), flags, device, _vp(stream)))
+
+
 ADAM_CLOCK_BYTES = 32     # sizeof(rg_adam_clock): int64 step, float neg_step_size, float bias2_sqrt, float step_f32, pad
 
 
@@ -353,6 +384,10 @@ class OptimTable:
         check(lib.rg_optim_create(C.byref(self._handle), device, n, _ptr_array(params, n), _ptr_array(grads, n),
                                   _ptr_array(state1, n), _ptr_array(state2, n), _ptr_array(copies, n),
                                   (C.c_int64 * max(n, 1))(*numels), (C.c_int * max(n, 1))(*grad_dtypes), a_cd))
+
+    def set_grad_scale_source(self, grad_scale_ptr: int) -> None:
+        """Later steps multiply the gradients by the float at this device address instead of ``grad_scale`` (0: off)."""
+        check(lib.rg_optim_set_grad_scale_source(self._handle, _vp(grad_scale_ptr or None)))
 
     @property
     def handle(self) -> int:

@@ -41,6 +41,7 @@ struct rg_plan {
   int xcd_write = 0;                 //   ... when every source sits on the line grid of its destination
   int xcd_write_offgrid = 256;       //   ... when some source does not (see fill_chunk_records)
   float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
+  const float* begun_scale_dev = nullptr;   // ... or where the kernels read it from (rg_step_begin_scaled)
   bool sums_describe_dst = false;   // the per-tensor sums on the device are those of the destinations as last written
   std::vector<TensorDesc> host_tensors;
   std::vector<int64_t> chunk_begin;  // [n_tensors + 1]
@@ -555,6 +556,27 @@ RG_API int rg_step_begin(rg_plan* p, float inv_scale, void* stream) {
   RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
   RG_HIP(launch_reduce(reduce_args(p, 0.0f, 0), p->n_chunks, s));
   p->begun_inv_scale = inv_scale;
+  p->begun_scale_dev = nullptr;
+  return RG_OK;
+}
+
+RG_API int rg_step_begin_scaled(rg_plan* p, const float* inv_scale_dev, void* stream) {
+  const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_step_begin_scaled");
+  if (rc != RG_OK) return rc;
+  p->sums_describe_dst = false;
+  if (inv_scale_dev == nullptr || (reinterpret_cast<uintptr_t>(inv_scale_dev) & 3u) != 0) {
+    set_error("rg_step_begin_scaled: inv_scale_dev must be a 4-byte aligned device pointer");
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(p->device);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  PassArgs a = pass_args(p, 1.0f);
+  a.scale_dev = inv_scale_dev;
+  a.xcd_run = p->xcd_reduce;
+  RG_HIP(launch_pass(kModeReduce, a, p->streaming, s));
+  RG_HIP(launch_reduce(reduce_args(p, 0.0f, 0), p->n_chunks, s));
+  p->begun_inv_scale = 1.0f;           // pending; the value itself is read on the device
+  p->begun_scale_dev = inv_scale_dev;
   return RG_OK;
 }
 
@@ -569,11 +591,13 @@ RG_API int rg_step_finish(rg_plan* p, float max_norm, int flags, void* stream) {
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   RG_HIP(launch_decide(reduce_args(p, max_norm, (flags & RG_STEP_IGNORE_OVERFLOW) ? 1 : 0), s));
   PassArgs a = pass_args(p, p->begun_inv_scale);
+  a.scale_dev = p->begun_scale_dev;
   a.result = p->d_result;
   a.write_on_overflow = (flags & RG_STEP_WRITE_ON_OVERFLOW) ? 1 : 0;
   split_for_write(p, a);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, s));
   p->begun_inv_scale = 0.0f;
+  p->begun_scale_dev = nullptr;
   return RG_OK;
 }
 

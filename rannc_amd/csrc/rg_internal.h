@@ -132,6 +132,7 @@ struct PassArgs {
   int32_t tile_elems;            // elements one block handles (== chunk_elems unless the pass splits chunks)
   int32_t tiles_per_chunk;       // blocks per chunk record
   float scale;
+  const float* scale_dev;        // non-null: the kernels read the scale from device memory instead of `scale`
   int32_t write_on_overflow;
   int32_t zero_fill;             // write pass: ignore the sources, store zeros
   int32_t norm_of_source;        // reduce pass: measure the source as stored (no rounding to dst)

@@ -292,7 +292,8 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
   char* dp = reinterpret_cast<char*>(rec.dst) + (size_t)start * (rec.dst_dtype == RG_F32 ? 4 : 2);
   const int src_kind = rec.src_dtype;
   const int dst_kind = a.norm_of_source ? rec.src_dtype : rec.dst_dtype;
-  const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale == 1.0f;   // never when accumulating
+  const float scale = a.scale_dev != nullptr ? *a.scale_dev : a.scale;   // a scale kept on the device (a loss scaler's state)
+  const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale_dev == nullptr && a.scale == 1.0f;   // never when accumulating
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   PendingStore pending{u32x4{0u, 0u, 0u, 0u}, nullptr, 0};
@@ -315,8 +316,8 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
     const bool has_head = ((MODE & kModeWrite) == 0 || PEEL) && (peeled & (peel - 1)) != 0;
 #define RG_PAIR(S, D)                                                                         \
   case S * 3 + D:                                                                             \
-    if (has_head) process_chunk<S, D, MODE, NT, T, true>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);  \
-    else process_chunk<S, D, MODE, NT, T, false>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);  \
+    if (has_head) process_chunk<S, D, MODE, NT, T, true>(sp, dp, len, scale, coef, raw_copy, acc, pending);  \
+    else process_chunk<S, D, MODE, NT, T, false>(sp, dp, len, scale, coef, raw_copy, acc, pending);  \
     break;
     switch (src_kind * 3 + dst_kind) {
       RG_PAIR(RG_F32, RG_F32)
@@ -328,8 +329,8 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
       RG_PAIR(RG_BF16, RG_F32)
       RG_PAIR(RG_BF16, RG_F16)
       default:
-        if (has_head) process_chunk<RG_BF16, RG_BF16, MODE, NT, T, true>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);
-        else process_chunk<RG_BF16, RG_BF16, MODE, NT, T, false>(sp, dp, len, a.scale, coef, raw_copy, acc, pending);
+        if (has_head) process_chunk<RG_BF16, RG_BF16, MODE, NT, T, true>(sp, dp, len, scale, coef, raw_copy, acc, pending);
+        else process_chunk<RG_BF16, RG_BF16, MODE, NT, T, false>(sp, dp, len, scale, coef, raw_copy, acc, pending);
         break;
     }
 #undef RG_PAIR

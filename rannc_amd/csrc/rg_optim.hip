@@ -51,6 +51,7 @@ struct OptArgs {
   const OptChunkRec* chunks;
   const StepResult* gate;
   const rg_adam_clock* clock;   // Adam only, optional: the step-dependent factors live on the device
+  const float* grad_scale_dev;  // optional: the gradient scale lives on the device (a loss scaler's 1 / scale)
   int32_t tile_elems;
   int32_t tiles_per_chunk;
   OptConst c;
@@ -204,6 +205,7 @@ __global__ __launch_bounds__(OptShape<ALGO>::kThreads) void optim_kernel(OptArgs
     if (a.gate->skipped != 0) return;
     coef = a.gate->coef;
   }
+  if (a.grad_scale_dev != nullptr) a.c.grad_scale = *a.grad_scale_dev;
   if (ALGO == kAdam && a.clock != nullptr) {
     // written by adam_clock_kernel earlier on the same stream
     a.c.neg_step_size = a.clock->neg_step_size;
@@ -254,6 +256,37 @@ __global__ void adam_clock_kernel(rg_adam_clock* clock, double lr, double beta1,
   clock->step_f32 = (float)step;
 }
 
+// One thread: the loss-scale schedule (see rg_scaler_update in ranncgrad.h).
+__global__ void scaler_init_kernel(rg_scaler_state* st, rg_scaler_state v) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  v.inv_scale = (float)(1.0 / (double)v.loss_scale);
+  *st = v;
+}
+
+__global__ void scaler_update_kernel(rg_scaler_state* st, const StepResult* result, int flags) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const bool dynamic = (flags & RG_SCALER_DYNAMIC) != 0;
+  float scale = st->loss_scale;
+  int unskipped = st->unskipped;
+  if (result->overflow != 0 && dynamic) {
+    scale = scale / 2.0f;
+    if (st->min_loss_scale > 0.0f && scale < st->min_loss_scale) scale = st->min_loss_scale;
+    if ((flags & RG_SCALER_TRUNCATE) != 0) scale = (float)(int)scale;
+    unskipped = 0;
+    st->skipped_steps = st->skipped_steps + 1;
+  } else {
+    unskipped += 1;
+  }
+  if (unskipped == st->scale_window && dynamic) {
+    scale = scale * st->scale_factor;
+    if (scale > st->max_loss_scale) scale = st->max_loss_scale;
+    unskipped = 0;
+  }
+  st->loss_scale = scale;
+  st->inv_scale = (float)(1.0 / (double)scale);
+  st->unskipped = unskipped;
+}
+
 }  // namespace
 }  // namespace rg
 
@@ -266,6 +299,7 @@ struct rg_optim {
   int64_t chunk_elems = RG_DEFAULT_CHUNK_ELEMS;
   int64_t total_numel = 0;
   bool has_state1 = false, has_state2 = false, any_copy = false;
+  const float* grad_scale_dev = nullptr;   // rg_optim_set_grad_scale_source
   struct Row {
     void* param;
     const void* grad;
@@ -467,6 +501,7 @@ static int launch_optim(const rg_optim* o, const OptConst& c, const rg_step_resu
   a.chunks = o->d_chunks;
   a.gate = reinterpret_cast<const StepResult*>(gate);
   a.clock = clock;
+  a.grad_scale_dev = o->grad_scale_dev;
   a.tile_elems = OptShape<ALGO>::kTileElems;
   a.tiles_per_chunk = (int32_t)((o->chunk_elems + OptShape<ALGO>::kTileElems - 1) / OptShape<ALGO>::kTileElems);
   a.c = c;
@@ -516,6 +551,15 @@ static int adam_step(rg_optim* o, const rg_adam_args* g, const rg_adam_clock* cl
   c.bias2_sqrt = (float)sqrt(bias2);
   c.eps = (float)g->eps;
   return launch_optim<kAdam>(o, c, g->gate, 30, stream, clock);
+}
+
+RG_API int rg_optim_set_grad_scale_source(rg_optim* o, const float* grad_scale_dev) {
+  if (o == nullptr || (reinterpret_cast<uintptr_t>(grad_scale_dev) & 3u) != 0) {
+    set_error("rg_optim_set_grad_scale_source: null table or a pointer that is not 4-byte aligned");
+    return RG_EINVAL;
+  }
+  o->grad_scale_dev = grad_scale_dev;
+  return RG_OK;
 }
 
 RG_API int rg_adam_step(rg_optim* o, const rg_adam_args* g, void* stream) {
@@ -575,4 +619,37 @@ RG_API int rg_sgd_step(rg_optim* o, const rg_sgd_args* g, void* stream) {
   c.first_step = g->first_step;
   c.has_momentum = g->momentum != 0.0 ? 1 : 0;
   return launch_optim<kSgd>(o, c, g->gate, c.has_momentum ? 22 : 14, stream);
+}
+
+RG_API int rg_scaler_init(rg_scaler_state* state_dev, const rg_scaler_state* init_host, int device, void* stream) {
+  if (state_dev == nullptr || init_host == nullptr || (reinterpret_cast<uintptr_t>(state_dev) & 3u) != 0) {
+    set_error("rg_scaler_init: null argument or a state that is not 4-byte aligned");
+    return RG_EINVAL;
+  }
+  if (!(init_host->loss_scale > 0.0f) || !(init_host->max_loss_scale > 0.0f) || !(init_host->min_loss_scale >= 0.0f) ||
+      init_host->scale_window < 1 || !(init_host->scale_factor > 1.0f)) {
+    set_error("rg_scaler_init: bad schedule (scale %g min %g max %g window %d factor %g)", init_host->loss_scale,
+              init_host->min_loss_scale, init_host->max_loss_scale, init_host->scale_window, init_host->scale_factor);
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(device);
+  hipLaunchKernelGGL(scaler_init_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), state_dev, *init_host);
+  RG_HIP(hipGetLastError());
+  return RG_OK;
+}
+
+RG_API int rg_scaler_update(rg_scaler_state* state_dev, const rg_step_result* result_dev, int flags, int device, void* stream) {
+  if (state_dev == nullptr || result_dev == nullptr || (reinterpret_cast<uintptr_t>(state_dev) & 3u) != 0) {
+    set_error("rg_scaler_update: null argument or a state that is not 4-byte aligned");
+    return RG_EINVAL;
+  }
+  if ((flags & ~(RG_SCALER_DYNAMIC | RG_SCALER_TRUNCATE)) != 0) {
+    set_error("rg_scaler_update: unknown flags %d", flags);
+    return RG_EINVAL;
+  }
+  DeviceGuard guard(device);
+  hipLaunchKernelGGL(scaler_update_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), state_dev,
+                     reinterpret_cast<const StepResult*>(result_dev), flags);
+  RG_HIP(hipGetLastError());
+  return RG_OK;
 }

@@ -156,6 +156,7 @@ class GradPlan {
 
   void fused_step(float inv_scale, float max_norm, int flags) { check(rg_fused_step(plan_.get(), inv_scale, max_norm, flags, plan_.stream())); }
   void step_begin(float inv_scale) { check(rg_step_begin(plan_.get(), inv_scale, plan_.stream())); }
+  void step_begin_scaled(uintptr_t inv_scale_dev) { check(rg_step_begin_scaled(plan_.get(), reinterpret_cast<const float*>(inv_scale_dev), plan_.stream())); }
   void step_finish(float max_norm, int flags) { check(rg_step_finish(plan_.get(), max_norm, flags, plan_.stream())); }
   void step_decide(float max_norm, int flags) { check(rg_step_decide(plan_.get(), max_norm, flags, plan_.stream())); }
   void unscale_pack(float inv_scale) { check(rg_unscale_pack(plan_.get(), inv_scale, plan_.stream())); }
@@ -662,6 +663,7 @@ void bind_registry(py::module_& m) {
       .def("sources", &GradPlan::sources)
       .def("fused_step", &GradPlan::fused_step, py::arg("inv_scale"), py::arg("max_norm"), py::arg("flags") = 0)
       .def("step_begin", &GradPlan::step_begin)
+      .def("step_begin_scaled", &GradPlan::step_begin_scaled, py::arg("inv_scale_device_ptr"))
       .def("step_finish", &GradPlan::step_finish, py::arg("max_norm"), py::arg("flags") = 0)
       .def("step_decide", &GradPlan::step_decide, py::arg("max_norm"), py::arg("flags") = 0)
       .def("unscale_pack", &GradPlan::unscale_pack)

@@ -50,6 +50,9 @@ class _FusedBase(torch.optim.Optimizer):
         self.gate: int = 0
         #: every gradient is multiplied by this first
         self.grad_scale: float = 1.0
+        #: device address of a float to multiply by instead (a loss scaler's ``1 / scale`` kept on the device,
+        #: ``rg_scaler_state.inv_scale``), so that a step recorded in a HIP graph follows the scale; 0: off
+        self.grad_scale_ptr: int = 0
         self._grad_sources: Dict[int, torch.Tensor] = {}
         self._feed = None                          # see set_grad_feed
         self._feed_params: List[torch.Tensor] = []
@@ -194,6 +197,13 @@ class _FusedBase(torch.optim.Optimizer):
                 known = self._native_lists[gi] = (params, len(params), _native.TensorList(params))
             known[2].clear_grads()
 
+    def _scale_source(self, table: _lib.OptimTable) -> _lib.OptimTable:
+        """Tell the table where the gradient scale lives, when that changed since its last launch."""
+        if getattr(table, "scale_source", 0) != self.grad_scale_ptr:
+            table.set_grad_scale_source(self.grad_scale_ptr)
+            table.scale_source = self.grad_scale_ptr
+        return table
+
     def _grad_of(self, p: torch.Tensor) -> Optional[torch.Tensor]:
         if self._feed is not None:
             self._sources_from_feed()
@@ -310,7 +320,7 @@ class FusedAdam(_FusedBase):
         b1, b2 = group["betas"]
         stream = stream_handle(dev)
         _lib.adam_clock_advance(clock.data_ptr(), group["lr"], b1, b2, self.gate, dev.index, stream)
-        table.adam_step_clocked(clock.data_ptr(), group["lr"], b1, b2, group["eps"], group["weight_decay"],
+        self._scale_source(table).adam_step_clocked(clock.data_ptr(), group["lr"], b1, b2, group["eps"], group["weight_decay"],
                                 decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
                                 gate=self.gate, stream=stream)
 
@@ -331,7 +341,7 @@ class FusedAdam(_FusedBase):
                 st.count += 1
                 st.steps_buf += 1
                 b1, b2 = group["betas"]
-                st.table.adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], st.count,
+                self._scale_source(st.table).adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], st.count,
                                    decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
                                    gate=self.gate, stream=stream_handle(st.device))
                 continue
@@ -365,7 +375,7 @@ class FusedAdam(_FusedBase):
                 vs = [self.state[p]["exp_avg_sq"] for p in ps]
                 table = self._table((gi, tuple(id(p) for p in ps)), ps, [grad_of[id(p)] for p in ps], ms, vs)
                 b1, b2 = group["betas"]
-                table.adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], step,
+                self._scale_source(table).adam_step(group["lr"], b1, b2, group["eps"], group["weight_decay"], step,
                                 decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
                                 gate=self.gate, stream=stream_handle(ps[0].device))
                 if len(by_step) == 1 and len(ps) == len(group["params"]):
@@ -405,7 +415,7 @@ class FusedSGD(_FusedBase):
             steady = self._steady_grads(gi, group)
             if steady is not None:
                 st, _ = steady
-                st.table.sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
+                self._scale_source(st.table).sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
                                   group["nesterov"], group["maximize"], first_step=False, grad_scale=self.grad_scale,
                                   gate=self.gate, stream=stream_handle(st.device))
                 continue
@@ -431,7 +441,7 @@ class FusedSGD(_FusedBase):
                     continue
                 bufs = [self.state[p]["momentum_buffer"] for p in ps] if group["momentum"] != 0 else None
                 table = self._table((gi, first, tuple(id(p) for p in ps)), ps, [grad_of[id(p)] for p in ps], bufs, None)
-                table.sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
+                self._scale_source(table).sgd_step(group["lr"], group["momentum"], group["dampening"], group["weight_decay"],
                                group["nesterov"], group["maximize"], first_step=first, grad_scale=self.grad_scale,
                                gate=self.gate, stream=stream_handle(ps[0].device))
                 if not first and not fresh and len(ps) == len(group["params"]):

@@ -151,6 +151,10 @@ class TensorPlan:
     def step_begin(self, inv_scale: float) -> None:
         self.plan.step_begin(inv_scale, self._stream())
 
+    def step_begin_scaled(self, inv_scale_ptr: int) -> None:
+        """``step_begin`` whose kernels read ``inv_scale`` from device memory (the loss scaler's state)."""
+        self.plan.step_begin_scaled(inv_scale_ptr, self._stream())
+
     def step_finish(self, max_norm: float, flags: int = _lib.RG_STEP_DEFAULT) -> None:
         self.plan.step_finish(max_norm, flags, self._stream())
 

@@ -246,3 +246,116 @@ def test_whole_optimizer_phase_replays_from_a_graph_with_a_skipped_step():
             x.copy_(opt.state[p]["exp_avg_sq"].cpu())
     assert steps_done == 4
     plan.close()
+
+
+def test_dynamic_loss_scale_on_the_device_replays_from_a_graph():
+    """The whole mixed-precision optimizer phase with a *dynamic* loss scale and no host read: the unscale reads
+    ``1 / scale`` from the scaler's state on the device (``rg_step_begin_scaled``), the clip decision and the Adam
+    step (device-resident count, gated) follow, then one thread applies the schedule (``rg_scaler_update``: halve
+    and truncate on overflow, double after ``scale_window`` clean steps).  Seven replays of one HIP graph - two with
+    an inf, two window doublings - against the oracle's ``patched_update_scale`` sequence and its Adam step."""
+    import ctypes
+    from oracle import gradpath as oracle
+    from oracle import optim as oracle_optim
+    from rannc_amd import _lib
+    from rannc_amd.fused_optim import FusedAdam
+    from rannc_amd.multi_tensor import stream_handle
+    dev = torch.device(DEV)
+    gen = torch.Generator().manual_seed(16)
+    shapes = [(20001,), (5,), (3000, 7)]
+    max_norm = 0.5
+    want_scaler = oracle.LossScalerState(loss_scale=25.0, unskipped=0, scale_window=2, min_loss_scale=None,
+                                         max_loss_scale=2.0 ** 24, dynamic=True)
+    masters_cpu = [torch.randn(s, generator=gen) for s in shapes]
+    m_cpu = [torch.zeros(s) for s in shapes]
+    v_cpu = [torch.zeros(s) for s in shapes]
+    masters = [torch.nn.Parameter(t.clone().to(DEV)) for t in masters_cpu]
+    models = [t.detach().to(torch.float16) for t in masters]
+    static_grads = [torch.zeros(s, dtype=torch.float16, device=DEV) for s in shapes]
+    bucket = [torch.zeros(s, device=DEV) for s in shapes]                 # never written on this route
+    plan = TensorPlan(static_grads, bucket)
+    state = torch.zeros(_lib.SCALER_STATE_BYTES // 4, dtype=torch.float32, device=DEV)
+    _lib.scaler_init(state.data_ptr(), 25.0, 0.0, 2.0 ** 24, 2, 2.0, 0, stream_handle(dev))
+    inv_ptr = state.data_ptr() + _lib.SCALER_INV_SCALE_OFFSET
+    opt = FusedAdam(masters, lr=1e-2, capturable=True)
+    opt.set_model_copies(masters, models)
+    opt.set_grad_sources(masters, static_grads)
+    opt.grad_scale_ptr = inv_ptr
+    opt.gate = plan.plan.result_device_ptr()
+
+    def phase():
+        s = stream_handle(dev)
+        plan.plan.step_begin_scaled(inv_ptr, s)
+        plan.plan.step_decide(max_norm, 0, s)
+        opt.step()
+        _lib.scaler_update(state.data_ptr(), plan.plan.result_device_ptr(), _lib.RG_SCALER_DYNAMIC | _lib.RG_SCALER_TRUNCATE, 0, s)
+
+    def device_scaler():
+        raw = state.cpu().numpy().tobytes()
+        return _lib.ScalerState.from_buffer_copy(raw)
+
+    def new_grads(scale, poison=False):
+        out = [(torch.randn(s, generator=gen) * 0.1 * scale).to(torch.float16) for s in shapes]
+        if poison:
+            out[0].view(-1)[77] = float("nan")
+        return out
+
+    steps_done = 0
+
+    def oracle_step(grads_cpu):
+        nonlocal steps_done
+        inv = 1.0 / want_scaler.loss_scale
+        want = oracle.fused_step(grads_cpu, ["f32"] * len(shapes), inv, max_norm)
+        skipped = oracle.patched_update_scale(want_scaler, bool(want.overflow))
+        assert skipped == bool(want.overflow)
+        if want.overflow:
+            return want
+        steps_done += 1
+        unscaled, _ = oracle.unscale_and_check(grads_cpu, inv)
+        if want.coef is not None:
+            unscaled = [u * torch.tensor(want.coef, dtype=torch.float32) for u in unscaled]
+        oracle_optim.adam_step(masters_cpu, unscaled, m_cpu, v_cpu, steps_done, lr=1e-2)
+        return want
+
+    g0 = new_grads(want_scaler.loss_scale)
+    for s, g in zip(static_grads, g0):
+        s.copy_(g)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        phase()                                                # eager: allocates the state and the tables
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    oracle_step(g0)
+    assert (device_scaler().loss_scale, device_scaler().unskipped) == (25.0, 1)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        phase()
+    scales_seen = []
+    # scale 25, one clean step done: clean -> 50 (window), inf -> 25, clean, inf -> 12 (12.5 truncated), clean, clean -> 24
+    for replay, poison in enumerate([False, True, False, True, False, False, False]):
+        gc = new_grads(want_scaler.loss_scale, poison)
+        for s, g in zip(static_grads, gc):
+            s.copy_(g)                                         # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle_step(gc)
+        res = plan.result()
+        got = device_scaler()
+        assert res.overflow == want.overflow == (1 if poison else 0) and res.skipped == res.overflow
+        assert (got.loss_scale, got.unskipped) == (float(want_scaler.loss_scale), want_scaler.unskipped), f"replay {replay}"
+        assert got.inv_scale == torch.tensor(1.0 / want_scaler.loss_scale, dtype=torch.float32).item()
+        scales_seen.append(got.loss_scale)
+        assert float(opt.state[masters[0]]["step"]) == float(steps_done)
+        for p, w, c in zip(masters, masters_cpu, models):
+            torch.testing.assert_close(p.detach().cpu(), w, rtol=2e-6, atol=2e-8, msg=f"replay {replay}")
+            assert_bits_equal(c.cpu(), p.detach().cpu().to(torch.float16), f"model copy, replay {replay}")
+        for p, w in zip(masters, masters_cpu):
+            w.copy_(p.detach().cpu())                          # continue from the GPU's trajectory
+        for p, w, x in zip(masters, m_cpu, v_cpu):
+            w.copy_(opt.state[p]["exp_avg"].cpu())
+            x.copy_(opt.state[p]["exp_avg_sq"].cpu())
+    assert scales_seen == [50.0, 25.0, 25.0, 12.0, 12.0, 24.0, 24.0]      # written by hand from the schedule
+    assert steps_done == 6 and device_scaler().skipped_steps == 2
+    plan.close()
