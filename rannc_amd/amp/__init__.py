@@ -59,6 +59,9 @@ class _CompiledStepPlan:
     def step_begin(self, inv_scale: float) -> None:
         self.gp.step_begin(inv_scale)
 
+    def step_begin_scaled(self, inv_scale_ptr: int) -> None:
+        self.gp.step_begin_scaled(inv_scale_ptr)
+
     def step_finish(self, max_norm: float, flags: int = 0) -> None:
         self.gp.step_finish(max_norm, flags)
 
@@ -147,6 +150,7 @@ class _AmpStash:
         # gradients and for adding fresh gradients onto stashed ones (gradient accumulation)
         self.fp32_unscale_plans = None
         self.fp32_accumulate_plans = None
+        self.device_scaler = None          # the LossScaler, when its schedule lives on the device
         self.compiled: Optional[_CompiledLists] = None     # made at the first steady-state exit of scale_loss
         self.feed = None                   # the GradPlan whose held gradients the pending write / step reads, if any
 
@@ -181,8 +185,45 @@ class LossScaler:
         self._max_loss_scale = max_loss_scale
         self._unskipped = 0
         self._has_overflow = False
+        # the schedule on the device (``amp.initialize(..., device_loss_scale=True)``): 32 bytes of state that the
+        # unscale, the optimizer step and a one-thread update kernel read and write; the host only looks on request
+        self.state: Optional[torch.Tensor] = None
+        self.update_flags = _lib.RG_SCALER_DYNAMIC
+
+    @property
+    def on_device(self) -> bool:
+        return self.state is not None
+
+    def to_device(self, device: torch.device) -> None:
+        """Write the schedule, as the attributes of this object describe it, into device memory (at set-up, and again
+        when those attributes were changed by hand)."""
+        if not self.dynamic:
+            raise ValueError("a static loss scale has no schedule to keep on the device")
+        from ..multi_tensor import stream_handle
+        if self.state is None:
+            self.state = torch.zeros(_lib.SCALER_STATE_BYTES // 4, dtype=torch.float32, device=device)
+        _lib.scaler_init(self.state.data_ptr(), float(self._loss_scale), float(self._min_loss_scale or 0.0),
+                         float(self._max_loss_scale), int(self._scale_seq_len), float(self._scale_factor),
+                         device.index or 0, stream_handle(device))
+        self.scale_on_device = self.state[0]            # 0-dim view: ``loss * scale`` without a host read
+
+    @property
+    def inv_scale_ptr(self) -> int:
+        return self.state.data_ptr() + _lib.SCALER_INV_SCALE_OFFSET
+
+    def device_state(self) -> "_lib.ScalerState":
+        """The schedule's state as the device holds it now (a host read: waits for the stream)."""
+        return _lib.ScalerState.from_buffer_copy(self.state.cpu().numpy().tobytes())
+
+    def update_on_device(self, result_ptr: int) -> None:
+        """Queue the schedule's update for the step whose flag is in the result block at ``result_ptr``."""
+        from ..multi_tensor import stream_handle
+        dev = self.state.device
+        _lib.scaler_update(self.state.data_ptr(), result_ptr, self.update_flags, dev.index or 0, stream_handle(dev))
 
     def loss_scale(self) -> float:
+        if self.state is not None:
+            return float(self.device_state().loss_scale)
         return self._loss_scale
 
     def clear_overflow_state(self) -> None:
@@ -216,20 +257,27 @@ class LossScaler:
             stash.unscale_plan = stash.unscale_cache.get_same_shapes("all", model_grads, master_grads, tune_new=not accumulate)
         else:
             stash.unscale_plan = stash.unscale_cache.get(model_grads, master_grads, tune_new=not accumulate)
-        inv = 1.0 / self._loss_scale
+        deferred = not accumulate and stash.fused and (stash.expect_clip or stash.optimizer_reads_model_grads)
+        # with the schedule on the device the deferred route never needs the scale on the host; the others do
+        inv = None if (self.on_device and deferred) else 1.0 / self.loss_scale()
         stash.sums_cover_all = False
         with torch.no_grad():
             if accumulate:
                 stash.unscale_plan.unscale_accumulate(inv)
-            elif stash.fused and (stash.expect_clip or stash.optimizer_reads_model_grads):
-                stash.unscale_plan.step_begin(inv)
+            elif deferred:
+                if inv is None:
+                    stash.unscale_plan.step_begin_scaled(self.inv_scale_ptr)
+                else:
+                    stash.unscale_plan.step_begin(inv)
                 stash.pending_finish = True
                 stash.pending_inv_scale = inv
                 stash.decided_max_norm = None
             else:
                 stash.unscale_plan.unscale_pack(inv)
                 stash.sums_cover_all = stash.fused
-        if self.dynamic:
+        if self.on_device:
+            stash._last_result, stash._last_result_plan = None, stash.unscale_plan     # the device decides; nobody waits
+        elif self.dynamic:
             stash.last_result = stash.unscale_plan.result()      # one host read, like the reference's .item()
             if stash.last_result.overflow:
                 self._has_overflow = True
@@ -261,7 +309,7 @@ class LossScaler:
 
 def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_level: str = "O2",
                loss_scale="dynamic", max_loss_scale: float = 2.0 ** 24, min_loss_scale: Optional[float] = None,
-               half_dtype: torch.dtype = torch.float16, fused: bool = True
+               half_dtype: torch.dtype = torch.float16, fused: bool = True, device_loss_scale: bool = False
                ) -> Tuple[torch.nn.Module, torch.optim.Optimizer]:
     """O2-style set-up: the model's floating-point parameters (batch-norm layers excepted)
     become ``half_dtype``; the optimizer is re-pointed at fp32 masters created as
@@ -280,7 +328,15 @@ def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_lev
     precision) the write never happens: ``clip_grad_norm`` only takes the clip decision on the
     device and ``optimizer.step`` reads the scaled model gradients, applies ``1/scale`` and the
     clip coefficient, updates the masters and writes the model copies in one kernel.  Anything
-    that looks at master gradients first writes them, and the step then takes them from memory."""
+    that looks at master gradients first writes them, and the step then takes them from memory.
+
+    ``device_loss_scale=True`` (dynamic scale, ``fused=True``, a ``FusedAdam`` / ``FusedAdamW`` - made ``capturable``
+    here): the loss scale and its schedule live in 32 bytes of device memory.  ``scale_loss`` multiplies the loss by
+    the scale where it is, the unscale and the optimizer step read ``1 / scale`` there, an overflow gates the step
+    on the device, and one thread updates the schedule after ``optimizer.step`` (Apex updates it at the context
+    exit; with one backward per step that is the same sequence).  Nothing in a training step then waits for the
+    device; ``scaler.loss_scale()`` and ``stash.last_result`` read it back on request.  Every stepped parameter
+    must be half precision (no fp32 batch-norm parameters)."""
     if opt_level != "O2":
         raise ValueError("only opt_level='O2' (fp32 masters for half parameters) is provided")
     bn = torch.nn.modules.batchnorm._BatchNorm
@@ -303,6 +359,17 @@ def initialize(model: torch.nn.Module, optimizer: torch.optim.Optimizer, opt_lev
     # RG_STEP_IGNORE_OVERFLOW makes the deferred write / the clip decision behave exactly like
     # ParamStorage::clipGradNorm on gradients that contain them (src/comp/ParamStorage.cpp:723-742).
     stash.step_flags = _lib.RG_STEP_DEFAULT if scaler.dynamic else _lib.RG_STEP_IGNORE_OVERFLOW
+    if device_loss_scale:
+        if not (scaler.dynamic and fused and stash.optimizer_reads_model_grads and hasattr(optimizer, "capturable")):
+            raise ValueError("device_loss_scale needs a dynamic loss scale, fused=True and a FusedAdam / FusedAdamW")
+        if any(p.dtype == torch.float32 for g in optimizer.param_groups for p in g["params"]):
+            raise ValueError("device_loss_scale: every parameter the optimizer steps on must be half precision")
+        if len(optimizer.state) and not optimizer.capturable:
+            raise ValueError("device_loss_scale: the optimizer already holds host-counted state; build it with capturable=True")
+        optimizer.capturable = True              # step counts on the device: a gated (skipped) step does not count
+        first = next(p for g in optimizer.param_groups for p in g["params"])
+        scaler.to_device(first.device)
+    stash.device_scaler = scaler if device_loss_scale else None
     _amp_state.loss_scalers = [scaler]
     _amp_state.opt_level = opt_level
     _patch_step(optimizer)
@@ -414,6 +481,42 @@ def _master_to_model(optimizer: torch.optim.Optimizer) -> None:
         stash.copy_back_plan.scale_cast(1.0)
 
 
+def _device_scaled_step(optimizer, stash: _AmpStash, old_step, args, kwargs):
+    """``optimizer.step`` with the loss-scale schedule on the device: the step kernel reads ``1 / scale`` and the clip
+    decision where they are and does nothing after an overflow; then one thread updates the schedule."""
+    scaler = stash.device_scaler
+    if not stash.pending_finish and stash.unscale_plan is None:
+        return old_step(*args, **kwargs)                 # no scale_loss has run: a plain step
+    result_ptr = stash.unscale_plan.plan.result_device_ptr()
+    if can_step_from_model_grads(optimizer) and not (args or kwargs) and stash.pending_inv_scale is None:
+        if stash.decided_max_norm is None:
+            decide_clip(optimizer, 0.0)
+        if stash.feed is not None:
+            optimizer.set_grad_feed(stash.feed, stash.pending_masters)
+        else:
+            optimizer.set_grad_sources(stash.pending_masters, stash.pending_model_grads)
+        optimizer.grad_scale_ptr, optimizer.gate = scaler.inv_scale_ptr, result_ptr
+        try:
+            ret = old_step()
+        finally:
+            optimizer.set_grad_sources([], [])
+            optimizer.grad_scale_ptr, optimizer.gate = 0, 0
+    else:
+        # the master gradients were looked at (or built up over several backward passes): they are in memory,
+        # unscaled; whether the step runs is then read from the device, as the host-side schedule would
+        finish_unscale(optimizer)
+        skipped = bool(stash.unscale_plan.result().skipped) or bool(scaler._has_overflow)
+        ret = None if skipped else old_step(*args, **kwargs)
+        scaler._has_overflow = False
+    scaler.update_on_device(result_ptr)
+    stash.pending_finish = False
+    stash.decided_max_norm = None
+    stash.unscale_plan.drop_sources()
+    stash.pending_model_grads = []
+    stash.feed = None
+    return ret
+
+
 def _patch_step(optimizer: torch.optim.Optimizer) -> None:
     stash = optimizer._amp_stash
     if stash.already_patched:
@@ -421,6 +524,8 @@ def _patch_step(optimizer: torch.optim.Optimizer) -> None:
     old_step = optimizer.step
 
     def new_step(*args, **kwargs):
+        if stash.device_scaler is not None:
+            return _device_scaled_step(optimizer, stash, old_step, args, kwargs)
         if getattr(stash, "skip_next_step", False):
             stash.skip_next_step = False
             stash.pending_finish = False
@@ -477,7 +582,7 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
             stashed_fp32[id(p)] = p.grad
             p.grad = None
     try:
-        yield loss.float() * scaler.loss_scale()
+        yield loss.float() * (scaler.scale_on_device if scaler.on_device else scaler.loss_scale())
     except BaseException:
         # the body failed: put the stashed gradients back (dropping a half-made scaled one) and let the error through
         for p in stash.all_fp32_from_fp32_params:
@@ -540,7 +645,6 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
     from ..param_storage import _PlanCache
     if stash.fp32_unscale_plans is None:
         stash.fp32_unscale_plans, stash.fp32_accumulate_plans = _PlanCache(), _PlanCache()
-    inv = 1.0 / scaler.loss_scale()
     fresh32, new32, old32 = [], [], []
     for p in stash.all_fp32_from_fp32_params:
         kept = stashed_fp32.get(id(p))
@@ -553,6 +657,8 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
             old32.append(kept)
             p.grad = kept                          # kept += new * inv below
     with torch.no_grad():
+        if fresh32 or new32:
+            inv = 1.0 / scaler.loss_scale()
         if fresh32:
             plan = stash.fp32_unscale_plans.get(fresh32, fresh32)
             plan.unscale_pack(inv)
@@ -563,9 +669,10 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
             plan.unscale_accumulate(inv)
             if scaler.dynamic and plan.result().overflow:       # a static scale never skips: nothing waits for the flag
                 scaler._has_overflow = True
-    should_skip = scaler.update_scale()
-    if should_skip:
-        stash.skip_next_step = True
+    if not scaler.on_device:                # on the device the schedule is updated after optimizer.step
+        should_skip = scaler.update_scale()
+        if should_skip:
+            stash.skip_next_step = True
     if not dropped_half_grads:
         for p in stash.all_fp16_params:       # Apex O2 drops the half grads once they are unscaled
             p.grad = None
@@ -654,6 +761,12 @@ def patch_amp_scaler():
     and reports that the step must be skipped."""
     scaler = _amp_state.loss_scalers[0]
     if getattr(scaler, "_rannc_patched", False):
+        return
+    if scaler.on_device:
+        # one rank: the sum of the flags is the flag and the minimum of int(loss_scale) is int(loss_scale) - the
+        # update kernel truncates the halved scale itself and zeroes its count of clean steps
+        scaler.update_flags |= _lib.RG_SCALER_TRUNCATE
+        scaler._rannc_patched = True
         return
     own_update = scaler.update_scale
 

@@ -719,3 +719,48 @@ def test_amp_named_master_params_completes_a_deferred_write(reader):
         assert len(gs) == len(ws) > 0
         for g, w in zip(gs, ws):
             assert_bits_equal(g, w, f"master gradient read through {reader} at step {step}")
+
+
+def test_amp_with_the_loss_scale_schedule_on_the_device():
+    """``amp.initialize(..., device_loss_scale=True)``: the same training loop with the schedule on the device and on
+    the host - an injected overflow in step 2 (skipped, scale halved and truncated by ``patch_amp_scaler``'s rule),
+    a window doubling - must walk the same parameters and the same scale sequence, and the device mode must not
+    read anything back unless asked."""
+    from rannc_amd.fused_optim import FusedAdam
+
+    def run(on_device):
+        torch.manual_seed(3)
+        model = _tiny_model()
+        opt = FusedAdam(model.parameters(), lr=1e-2)
+        model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 7, min_loss_scale=None,
+                                    device_loss_scale=on_device)
+        scaler = amp._amp_state.loss_scalers[0]
+        scaler._loss_scale, scaler._scale_seq_len = 100.0, 3
+        if on_device:
+            scaler.to_device(torch.device(DEV))           # rewrite the device state from the edited attributes
+        rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+        gen = torch.Generator().manual_seed(4)
+        scales = []
+        for step in range(7):
+            x = torch.randn(16, 32, generator=gen).to(DEV).to(torch.float16)
+            loss = rm(x).float().pow(2).mean()
+            with amp.scale_loss(loss, opt) as scaled:
+                scaled.backward()
+                if step == 2:
+                    opt._amp_stash.all_fp16_params[1].grad.view(-1)[0] = float("inf")
+            rm.clip_grad_norm(1.0)
+            opt.step()
+            opt.zero_grad()
+            scales.append(scaler.loss_scale())
+        masters = [m.detach().cpu().clone() for m in opt._amp_stash.all_fp32_from_fp16_params]
+        steps = float(opt.state[opt._amp_stash.all_fp32_from_fp16_params[0]]["step"])
+        return scales, masters, steps
+
+    host_scales, host_masters, host_steps = run(False)
+    dev_scales, dev_masters, dev_steps = run(True)
+    # 100: clean, clean, inf -> int(50) = 50, then three clean steps -> 100, one more clean
+    assert host_scales == [100.0, 100.0, 50.0, 50.0, 50.0, 100.0, 100.0]
+    assert dev_scales == host_scales
+    assert host_steps == dev_steps == 6.0
+    for a, b in zip(dev_masters, host_masters):
+        torch.testing.assert_close(a, b, rtol=2e-6, atol=1e-8)
