@@ -48,6 +48,8 @@ def parse_args():
     ap.add_argument("--chunk-elems", type=int, default=0)
     ap.add_argument("--c5-elements", type=int, default=10_000_000_000, help="total elements of the ZeRO flat buffer")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--loss-scale", default="static", choices=("static", "dynamic", "dynamic_device"),
+                    help="--op api_step: where the loss scale lives")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain elementwise kernels over 1 GiB of fp32 first (out = in * 1.5: 1 GiB read, "
                          "1 GiB written; known traffic for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -638,11 +640,13 @@ def cpu_baseline_optimizer(op: str, shapes, seed: int, budget_s: float, bytes_pe
 
 # ----------------------------------------------------------------------------- the drop-in API path
 
-def bench_api_step(args, key: str) -> dict:
-    full = _api_step_leg(args, key, 1.0)
+def bench_api_step(args, key: str, scale_mode: str = "static") -> dict:
+    """``scale_mode``: "static" (a fixed loss scale: nothing is read back), "dynamic" (the schedule on the host: one
+    read of the overflow flag per step, as the reference does) or "dynamic_device" (the schedule on the device)."""
+    full = _api_step_leg(args, key, 1.0, scale_mode)
     # the same tensor list with every tensor cut to one row: the kernels have next to nothing to do, so the wall
     # time of a step is the host's own cost of driving the API (including its one wait for the flag per step)
-    tiny = _api_step_leg(args, key, 0.0)
+    tiny = _api_step_leg(args, key, 0.0, scale_mode)
     full["host_only"] = {"what": "same calls on the same tensor list with every tensor cut to one row of dim 0",
                          "elements": tiny["config"]["elements"], "us_per_step": tiny["value"],
                          "device_us_per_step": tiny["device_us_per_step"], "us_per_call": tiny["host_us_per_call"]}
@@ -651,7 +655,7 @@ def bench_api_step(args, key: str) -> dict:
     return full
 
 
-def _api_step_leg(args, key: str, scale_numel: float) -> dict:
+def _api_step_leg(args, key: str, scale_numel: float, scale_mode: str = "static") -> dict:
     """Host time of the path a training script drives, on a parameter list shaped like ``key``: the exit of
     ``amp.scale_loss`` (unscale + flag), ``RaNNCModule.clip_grad_norm``, ``FusedAdam.step`` and ``zero_grad``.
     Backward is replaced by handing every half parameter a ready gradient tensor.  Reports wall microseconds per
@@ -679,7 +683,9 @@ def _api_step_leg(args, key: str, scale_numel: float) -> dict:
 
     model = Holder()
     opt = FusedAdam(model.parameters(), lr=1e-4)
-    model, opt = amp.initialize(model, opt, opt_level="O2", half_dtype=half, loss_scale=65536.0)
+    model, opt = amp.initialize(model, opt, opt_level="O2", half_dtype=half,
+                                loss_scale=65536.0 if scale_mode == "static" else "dynamic",
+                                device_loss_scale=scale_mode == "dynamic_device")
     rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
     rm._deploy()
     params = list(model.parameters())
@@ -742,13 +748,14 @@ def _api_step_leg(args, key: str, scale_numel: float) -> dict:
         "ms_per_step": round(wall * 1e3, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 model / f32 masters", "data": "synthetic",
         "config": {"workload": key, "op": "api_step", "tensors": len(params), "elements": n, "seed": args.seed,
-                   "deferred_write": bool(stash.fused), "optimizer": "FusedAdam"},
+                   "deferred_write": bool(stash.fused), "optimizer": "FusedAdam", "loss_scale": scale_mode},
         "device_us_per_step": round(dev_s * 1e6, 1),
         "host_us_per_call": {k: round(v / args.steps * 1e6, 1) for k, v in host.items()},
         "host_us_per_step_without_assign": round(sum(v for k, v in host.items() if k != "assign_grads") / args.steps * 1e6, 1),
         "algorithmic_bytes_per_step": bytes_per_elem * n,
         "GB/s": round(bytes_per_elem * n / wall / 1e9, 1),
-        "note": "scale_loss_exit includes the wait for the overflow flag (one host read per step, as the reference's .item())",
+        "note": "with loss_scale 'dynamic' scale_loss_exit includes the wait for the overflow flag (one host read per step, "
+                "as the reference's .item()); 'static' and 'dynamic_device' read nothing back",
     }
     rm.undeploy()
     del model, opt, rm, params, grads
@@ -909,7 +916,7 @@ def main() -> int:
         return 0
 
     if args.op == "api_step":
-        print(json.dumps(bench_api_step(args, args.workload or "c4_resnet152x2")), flush=True)
+        print(json.dumps(bench_api_step(args, args.workload or "c4_resnet152x2", args.loss_scale)), flush=True)
         return 0
 
     clocks = gpu_clocks()
@@ -974,10 +981,13 @@ def main() -> int:
             configs.append({"workload": "c2_bert_large", "op": op3, "ms_per_step": r["ms_per_step"], "GB/s": r["value"],
                             "pct_of_hbm_peak": r["pct_of_hbm_peak"], "bytes_per_elem": r["config"]["bytes_per_elem"],
                             "roofline": r["roofline"], "steps": sub})
-        for k3 in ("c4_resnet152x2", "c2_bert_large"):
+        for k3, mode in (("c4_resnet152x2", "static"), ("c2_bert_large", "static"), ("c1_mlp", "static"),
+                         ("c4_resnet152x2", "dynamic"), ("c4_resnet152x2", "dynamic_device"),
+                         ("c1_mlp", "dynamic"), ("c1_mlp", "dynamic_device")):
             sub_args = argparse.Namespace(**dict(vars(args), op="api_step", steps=max(args.steps, 30)))
-            r = bench_api_step(sub_args, k3)
-            configs.append({"workload": k3, "op": "api_step", "what": "scale_loss exit + clip_grad_norm + FusedAdam.step + zero_grad "
+            r = bench_api_step(sub_args, k3, mode)
+            configs.append({"workload": k3, "op": "api_step", "loss_scale": mode,
+                            "what": "scale_loss exit + clip_grad_norm + FusedAdam.step + zero_grad "
                             "through RaNNCModule / amp, wall time per training step",
                             "us_per_step": r["value"], "device_us_per_step": r["device_us_per_step"],
                             "host_only_us_per_step": r["host_us_per_step"], "host_us_per_call": r["host_only"]["us_per_call"],

@@ -772,6 +772,13 @@ def patch_amp_scaler():
 
     def update_scale_on_all_ranks():
         overflowed_here = own_update()
+        if _pyrannc.get_world_size() == 1:
+            # one rank: the sum of the flags is the flag and the minimum of int(loss_scale) is int(loss_scale);
+            # the reference's two device round trips per step (a .cuda() and an .item()) have nothing to exchange
+            if overflowed_here:
+                scaler._loss_scale = int(scaler._loss_scale)
+                scaler._unskipped = 0
+            return overflowed_here
         flag = torch.tensor([1 if overflowed_here else 0], dtype=torch.int32).cuda()
         _allreduce_sum(flag)
         if flag.item() == 0:

@@ -288,11 +288,25 @@ class FusedAdam(_FusedBase):
         params = group["params"]
         if not params:
             return
+        clock = self._clocks.get(gi)
+        steady = self._steady_grads(gi, group) if clock is not None else None
+        if steady is not None:
+            # same parameters, all with usable gradients, as at the step that made the record: the table is in place
+            # (re-pointed at the gradients by _steady_grads), only the two launches remain
+            st, _ = steady
+            b1, b2 = group["betas"]
+            stream = stream_handle(st.device)
+            _lib.adam_clock_advance(clock.data_ptr(), group["lr"], b1, b2, self.gate, st.device.index, stream)
+            self._scale_source(st.table).adam_step_clocked(clock.data_ptr(), group["lr"], b1, b2, group["eps"],
+                                                           group["weight_decay"], decoupled=self._decoupled,
+                                                           maximize=group["maximize"], grad_scale=self.grad_scale,
+                                                           gate=self.gate, stream=stream)
+            return
+        self._steady.pop(gi, None)
         grads = [self._grad_of(p) for p in params]
         if any(g is None for g in grads):
             raise RuntimeError("a capturable optimizer needs a gradient for every parameter at every step")
         dev = params[0].device
-        clock = self._clocks.get(gi)
         if clock is None:
             counts = set()
             for p, g in zip(params, grads):
@@ -323,6 +337,7 @@ class FusedAdam(_FusedBase):
         self._scale_source(table).adam_step_clocked(clock.data_ptr(), group["lr"], b1, b2, group["eps"], group["weight_decay"],
                                 decoupled=self._decoupled, maximize=group["maximize"], grad_scale=self.grad_scale,
                                 gate=self.gate, stream=stream)
+        self._make_steady(gi, group, table, grads, None)
 
     @torch.no_grad()
     def step(self, closure=None):
