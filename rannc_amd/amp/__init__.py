@@ -230,7 +230,7 @@ class LossScaler:
         self._has_overflow = False
 
     def unscale(self, stash: _AmpStash, model_grads: List[torch.Tensor], master_grads: List[torch.Tensor],
-                accumulate: bool = False, all_params: bool = False, plan=None) -> None:
+                accumulate: bool = False, all_params: bool = False, plan=None, covers_all: bool = False) -> None:
         """``master_grad = float(model_grad) * (1 / scale)`` for every pair in one launch, with the
         inf/NaN flag and - for free - the gradient norm.  In fused mode only the read pass runs
         here; the values are written by ``finish_unscale``.  ``accumulate`` adds to the master
@@ -263,7 +263,10 @@ class LossScaler:
         stash.sums_cover_all = False
         with torch.no_grad():
             if accumulate:
+                # one pass: unscale, flag, add, and the sums of the *results* - when the pass covers every master
+                # gradient, clip_grad_norm needs no pass of its own to know the norm (clip_from_unscale_sums)
                 stash.unscale_plan.unscale_accumulate(inv)
+                stash.sums_cover_all = stash.fused and covers_all
             elif deferred:
                 if inv is None:
                     stash.unscale_plan.step_begin_scaled(self.inv_scale_ptr)
@@ -640,7 +643,8 @@ def scale_loss(loss: torch.Tensor, optimizer: torch.optim.Optimizer):
             masters.append(m)
         stash.pending_masters, stash.pending_model_grads = masters, list(model_grads)
         if model_grads:
-            scaler.unscale(stash, model_grads, master_grads, accumulate=accumulate)
+            scaler.unscale(stash, model_grads, master_grads, accumulate=accumulate,
+                           covers_all=len(model_grads) == len(half_params))
     # fp32 parameters keep their own .grad; it carries the loss scale too
     from ..param_storage import _PlanCache
     if stash.fp32_unscale_plans is None:

@@ -764,3 +764,56 @@ def test_amp_with_the_loss_scale_schedule_on_the_device():
     assert host_steps == dev_steps == 6.0
     for a, b in zip(dev_masters, host_masters):
         torch.testing.assert_close(a, b, rtol=2e-6, atol=1e-8)
+
+
+@pytest.mark.parametrize("micro_batches", [2, 4])
+@pytest.mark.parametrize("fused", [False, True])
+def test_amp_gradient_accumulation_then_clip(micro_batches, fused):
+    """Accumulation steps {2, 4} as the reference's tests run them (``test/test_simple.py:21-46``,
+    ``test/common.py:98-103``), followed by ``clip_grad_norm``: the accumulated master gradients are the oracle's
+    (bit for bit) and the clip multiplies them by the coefficient of their norm.  In fused mode the norm comes from
+    the sums the accumulating pass left on the device - ``clip_grad_norm`` makes no pass over the gradients unless
+    it clips - in eager mode from a pass of its own; both within 1e-6 of the oracle's."""
+    model = _tiny_model()
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    model, opt = amp.initialize(model, opt, opt_level="O2", max_loss_scale=2.0 ** 8, fused=fused)
+    rm = rannc_amd.RaNNCModule(model, opt, enable_apex_amp=True)
+    want = None
+    for i in range(micro_batches):
+        x = torch.randn(16, 32, device=DEV, dtype=torch.float16)
+        loss = rm(x).float().pow(2).mean()
+        with amp.scale_loss(loss, opt) as scaled:
+            scaled.backward()
+            grads = [p.grad.detach().cpu().clone() for p in opt._amp_stash.all_fp16_params]
+        if want is None:
+            want, _ = oracle.unscale_and_check(grads, 1.0 / 256.0)
+        else:
+            oracle.unscale_accumulate(want, grads, 1.0 / 256.0)
+    stash = opt._amp_stash
+    masters = stash.all_fp32_from_fp16_params
+    for m, w in zip(masters, want):
+        assert_bits_equal(m.grad.cpu(), w, "accumulated master grad")
+    assert stash.sums_cover_all == fused                  # the accumulating pass's sums are kept for the clip
+    norm = oracle.grad_global_l2_norm(want)
+    max_norm = 0.5 * norm                                 # clips
+    rm.clip_grad_norm(max_norm)
+    if fused:
+        assert stash.clip_decided and not stash.sums_cover_all        # took the decision from the sums
+        res = stash.unscale_plan.result()
+        assert res.clipped == 1 and math.isclose(res.norm, norm, rel_tol=1e-6)
+        coef = res.coef
+    else:
+        coef = None
+    clipped = [w.clone() for w in want]
+    _, want_coef = oracle.clip_grad_norm(clipped, float(torch.tensor(max_norm, dtype=torch.float32)))
+    assert want_coef is not None
+    if coef is None:
+        coef = float(torch.tensor(want_coef, dtype=torch.float32))
+        for m, w in zip(masters, clipped):
+            torch.testing.assert_close(m.grad.cpu(), w, rtol=2e-6, atol=0)
+    else:
+        assert math.isclose(coef, want_coef, rel_tol=1e-6)
+        for m, w in zip(masters, want):
+            assert_bits_equal(m.grad.cpu(), w * torch.tensor(coef, dtype=torch.float32), "clipped with the device's coefficient")
+    opt.step()
+    opt.zero_grad()
