@@ -374,26 +374,35 @@ def run_host_layer_op(w: StepWorkload, op: str, steps: int, warmup: int) -> dict
     for i, p in enumerate(params):
         st.register_param(id(p), p)
         ids[f"p{i:05d}"] = id(p)
+    try:
+        from rannc_amd import _ranncgrad
+        owners, fresh = _ranncgrad.TensorList(params), _ranncgrad.TensorList(w.grads)
+        hand_out = lambda: owners.set_grads(fresh)        # as backward does: from C++
+    except ImportError:
+        def hand_out():
+            for p, g in zip(params, w.grads):
+                p.grad = g
     if op == "consolidate":
         con = GradConsolidation(st, [id(p) for p in params], False, False)
 
         def fn():
-            for p, g in zip(params, w.grads):      # backward left fresh gradients outside the buckets
-                p.grad = g
+            hand_out()                             # backward left fresh gradients outside the buckets
             con.consolidate()
         nbytes, kernel = 2 * s * n, "pass_kernel<write> (raw copy)"
     else:
-        st.deploy("g", ids, enable_zero=True, allreduce_amp_master_params=True)
+        from rannc_amd import _pyrannc
+        mod = _pyrannc.RaNNCModule(True, True, True)       # amp masters reduced in fp32, ZeRO: the product's path
+        mod.init({k: params[i] for i, k in enumerate(ids)}, False)
         for p, g in zip(params, w.grads):
             p.grad = g
         wide = 4 if w.grads[0].dtype == torch.float16 else s       # the reference widens fp16 only (ParamStorage.cpp:483-486)
 
         def fn():
-            st.allreduce_param_grads_zero("g")
+            mod.allreduce_grads_zero()
         nbytes, kernel = 2 * (s + wide) * n, "pass_kernel<write> x2 (pack into staging, copy back)"
     wall, dev_s = timed(fn, steps, warmup, 10)
     if op != "consolidate":
-        st.undeploy("g")
+        mod.undeploy()
     return entry(w.key, op, wall, nbytes, roofline(kernel, nbytes, dev_s, None,
                  note="launch time = all launches of the operation (device events); ms_per_step is wall time including "
                       "the host's per-parameter bookkeeping"), steps=steps, tensors=len(params))

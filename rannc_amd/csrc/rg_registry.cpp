@@ -195,6 +195,53 @@ class GradPlan {
   bool rebuilt_ = false;
 };
 
+// ------------------------------------------------------------------------------------------------ GradBuckets
+
+// The per-step half of GradConsolidation (src/comp/ParamStorage.cpp:154-176) for parameters whose gradients live in
+// their own buckets: `views[i]` is parameter i's slice of its dtype's bucket.  consolidate() makes every .grad that
+// view - a gradient that lives elsewhere is copied in, a missing one starts from zeros - with one copy launch and
+// one zero launch for all parameters, instead of the reference's copy_ / zero_ per parameter.
+class GradBuckets {
+ public:
+  GradBuckets(std::shared_ptr<TensorList> params, std::shared_ptr<TensorList> views) : params_(std::move(params)), views_(std::move(views)) {
+    if (params_->size() != views_->size()) throw std::invalid_argument("one bucket view per parameter");
+  }
+  // returns (gradients copied in, views zeroed)
+  std::pair<int, int> consolidate() {
+    const auto& views = views_->tensors();
+    std::vector<at::Tensor> copy_src, copy_dst, zero_src, zero_dst;
+    auto& params = const_cast<std::vector<at::Tensor>&>(params_->tensors());
+    for (size_t i = 0; i < params.size(); ++i) {
+      at::Tensor& p = params[i];
+      const at::Tensor& view = views[i];
+      const at::Tensor& g = p.grad();
+      if (g.defined()) {
+        if (g.data_ptr() == view.data_ptr()) continue;                       // :158-160
+        copy_src.push_back(g.is_contiguous() ? g : g.contiguous());
+        copy_dst.push_back(view);
+        p.mutable_grad() = view;                                             // :163-166
+      } else {
+        p.mutable_grad() = view;                                             // :169-175
+        zero_src.emplace_back();
+        zero_dst.push_back(view);
+      }
+    }
+    if (!copy_src.empty()) {
+      copy_plan_.bind(copy_src, copy_dst);
+      check(rg_scale_cast(copy_plan_.get(), 1.0f, copy_plan_.stream()));
+    }
+    if (!zero_dst.empty()) {
+      zero_plan_.bind(zero_src, zero_dst);
+      check(rg_zero(zero_plan_.get(), zero_plan_.stream()));
+    }
+    return {(int)copy_src.size(), (int)zero_dst.size()};
+  }
+
+ private:
+  std::shared_ptr<TensorList> params_, views_;
+  PairPlan copy_plan_, zero_plan_;
+};
+
 // ------------------------------------------------------------------------------------------------ ParamStorage
 
 struct SegmentLayout {
@@ -309,6 +356,33 @@ class ParamStorage {
   // the gradient (:419-427).  Two launches for all parameters; the buffers persist (BufferTensorCache).
   std::vector<at::Tensor> allreduce_param_grads_zero(const std::string& gid) {
     Graph& g = graph(gid);
+    // The steady state - the same parameters hold gradients at the same addresses as last time - is two launches
+    // over the tables of last time; anything else walks the parameters and rebinds them.
+    if (g.stage_valid && g.stage_generation == generation_) {
+      size_t k = 0;
+      bool same = true;
+      for (long pid : g.sorted) {
+        const at::Tensor& param = get_param_tensor(pid);
+        const at::Tensor& grad = param.grad();
+        if (!param.requires_grad() || !grad.defined()) continue;
+        if (k >= g.stage_grad_ptrs.size() || grad.data_ptr() != g.stage_grad_ptrs[k] || grad.numel() != g.stage_grad_numel[k] ||
+            !grad.is_contiguous()) {
+          same = false;
+          break;
+        }
+        ++k;
+      }
+      if (same && k == g.stage_grad_ptrs.size()) {
+        if (k > 0) {
+          check(rg_scale_cast(g.stage_pack.get(), 1.0f, g.stage_pack.stream()));
+          check(rg_scale_cast(g.stage_back.get(), 1.0f, g.stage_back.stream()));
+        }
+        return g.stage_bufs;
+      }
+    }
+    g.stage_valid = false;
+    g.stage_grad_ptrs.clear();
+    g.stage_grad_numel.clear();
     std::vector<at::Tensor> srcs, dsts, back_src, back_dst, bufs;
     for (long pid : g.sorted) {
       const at::Tensor& param = get_param_tensor(pid);
@@ -331,6 +405,8 @@ class ParamStorage {
       back_src.push_back(buf.narrow(0, 0, n));
       back_dst.push_back(flat);
       bufs.push_back(buf);
+      g.stage_grad_ptrs.push_back(grad.data_ptr());
+      g.stage_grad_numel.push_back(n);
     }
     if (!srcs.empty()) {
       g.stage_pack.bind(srcs, dsts);
@@ -338,6 +414,9 @@ class ParamStorage {
       g.stage_back.bind(back_src, back_dst);
       check(rg_scale_cast(g.stage_back.get(), 1.0f, g.stage_back.stream()));
     }
+    g.stage_bufs = bufs;
+    g.stage_valid = true;
+    g.stage_generation = generation_;
     return bufs;
   }
 
@@ -465,6 +544,12 @@ class ParamStorage {
     std::unique_ptr<GradPlan> selected_plan[2], scale_plan[2], zero_plan;
     uint64_t selected_generation[2] = {0, 0}, scale_generation = 0, zero_generation = 0;
     PairPlan stage_pack, stage_back;
+    // what the last allreduce_param_grads_zero bound: the gradients' addresses and sizes, the staging buffers
+    std::vector<const void*> stage_grad_ptrs;
+    std::vector<int64_t> stage_grad_numel;
+    std::vector<at::Tensor> stage_bufs;
+    bool stage_valid = false;
+    uint64_t stage_generation = 0;
   };
 
   Graph& graph(const std::string& gid) {
@@ -681,6 +766,10 @@ void bind_registry(py::module_& m) {
       .def("close", &GradPlan::close)
       .def_property_readonly("num_chunks", &GradPlan::num_chunks)
       .def_property_readonly("handle", &GradPlan::handle);
+
+  py::class_<GradBuckets>(m, "GradBuckets")
+      .def(py::init<std::shared_ptr<TensorList>, std::shared_ptr<TensorList>>(), py::arg("params"), py::arg("views"))
+      .def("consolidate", &GradBuckets::consolidate);
 
   py::class_<ParamStorage, std::shared_ptr<ParamStorage>>(m, "ParamStorage")
       .def(py::init<>())

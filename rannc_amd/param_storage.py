@@ -21,6 +21,11 @@ import torch
 from . import _lib
 from .multi_tensor import TensorPlan, dtype_code, fill_zero_
 
+try:        # the compiled module: per-step loops over parameters in C++
+    from . import _ranncgrad as _native
+except ImportError:
+    _native = None
+
 _DTYPE_ORDER = (torch.float32, torch.float16, torch.bfloat16)
 
 
@@ -165,6 +170,7 @@ class GradConsolidation:
                 self.amp_grad_tensors_next[pid] = self.grad_tensors[pid]
         self._copy_plan = _PlanCache()
         self._zero_plan = _PlanCache()
+        self._compiled: Dict[int, object] = {}     # id of a view map -> the compiled module's GradBuckets over it
 
     def consolidate(self) -> None:
         """``GradConsolidation::consolidate`` (``src/comp/ParamStorage.cpp:118-179``): swap the
@@ -176,6 +182,18 @@ class GradConsolidation:
             cur = self.consolidated_grads[torch.float32]
             self.consolidated_grads[torch.float32] = self.consolidated_amp_fp32_next
             self.consolidated_amp_fp32_next = cur
+        if _native is not None and not self.consolidate_master_params:
+            # the walk over the parameters in C++ (two launches at most); one object per view map, since the two
+            # fp32 buckets of an amp run swap places at every call
+            buckets = self._compiled.get(id(self.grad_tensors))
+            if buckets is None:
+                params = [self.storage.get_param_tensor(pid) for pid in self.param_ids]
+                views = [self.grad_tensors[pid] for pid in self.param_ids]
+                buckets = self._compiled[id(self.grad_tensors)] = _native.GradBuckets(_native.TensorList(params),
+                                                                                      _native.TensorList(views))
+            with torch.no_grad():
+                buckets.consolidate()
+            return
         copy_src: List[torch.Tensor] = []
         copy_dst: List[torch.Tensor] = []
         zero_dst: List[torch.Tensor] = []
