@@ -272,7 +272,14 @@ class FusedAdam(_FusedBase):
         0-dim float32 GPU tensor), nothing about a step is decided on the host, and ``step()`` may be recorded in
         a HIP graph and replayed.  Every parameter of a group must then have a gradient at every step, at the same
         address (graph capture needs that anyway), and the first ``step()`` - which allocates the state - has to
-        run outside a capture."""
+        run outside a capture.
+
+        What a capture freezes: ``lr``, ``betas``, ``eps``, ``weight_decay`` and ``maximize`` of every group, and
+        ``grad_scale`` when it is passed by value, are kernel arguments and so become part of the recorded graph -
+        changing ``param_groups[i]["lr"]`` afterwards affects eager steps only, a replayed graph keeps the values
+        of the capture (record a new graph after a learning-rate change).  What a replay does follow, because it
+        is read from device memory: the step count and its bias corrections, the gate (clip coefficient, skip)
+        and, with ``grad_scale_ptr``, 1 / loss scale."""
         if lr < 0 or eps < 0 or not 0 <= betas[0] < 1 or not 0 <= betas[1] < 1 or weight_decay < 0:
             raise ValueError("invalid Adam hyper-parameters")
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, maximize=maximize))
