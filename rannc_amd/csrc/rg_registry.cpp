@@ -299,7 +299,10 @@ class ParamStorage {
   std::vector<long> sorted_param_ids(const std::string& gid) { return graph(gid).sorted; }
   bool zero_enabled(const std::string& gid) { return graph(gid).zero; }
   // buckets the gradients of this graph are views of (GradConsolidation); clear_param_grads then clears those
-  void set_consolidated_grads(const std::string& gid, const std::vector<at::Tensor>& buckets) { graph(gid).buckets = buckets; }
+  void set_consolidated_grads(const std::string& gid, const std::vector<at::Tensor>& buckets) {
+    for (size_t i = 0; i < buckets.size(); ++i) require_gpu_contiguous(buckets[i], "bucket", i);
+    graph(gid).buckets = buckets;
+  }
 
   // ---- per-step operations
   // calcGradGlobalL2Norm (src/comp/ParamStorage.cpp:747-819): one read-only launch over all gradients in name
@@ -308,6 +311,7 @@ class ParamStorage {
     GradPlan& plan = selected_plan(gid, use_amp_master);
     if (plan.bind() <= 0) return 0.0;
     plan.grad_norm();
+    plan.drop_sources();   // queued: PyTorch's allocator is stream-ordered, so the gradients may be freed from here on
     return plan.raw_result().norm;
   }
   // clipGradNorm (:721-745): decided and applied on the device without a host round trip.
@@ -315,6 +319,7 @@ class ParamStorage {
     GradPlan& plan = selected_plan(gid, use_amp_master);
     if (plan.bind() <= 0) return;
     plan.fused_step(1.0f, max_grad_norm, RG_STEP_IGNORE_OVERFLOW);
+    plan.drop_sources();
   }
   // doScaleGrads (:598-615): grad *= 1/world or grad *= world
   void do_scale_grads(const std::string& gid, bool unscale, bool amp_master_grads, int world_size) {
@@ -330,6 +335,7 @@ class ParamStorage {
     if (slot->bind() <= 0) return;
     const float ratio = 1.0f / (float)world_size;
     slot->scale_cast(unscale ? 1.0f / ratio : ratio);
+    slot->drop_sources();
   }
   // clearParamGrads (:540-557)
   void clear_param_grads(const std::string& gid) {
@@ -348,6 +354,7 @@ class ParamStorage {
     }
     if (g.zero_plan->bind() <= 0) return;
     g.zero_plan->zero();
+    g.zero_plan->drop_sources();
   }
 
   // allReduceParamGradsZero (:440-520) for a group of one: every defined gradient is packed (cast to fp32 for
@@ -673,10 +680,10 @@ class RaNNCModule {
     require();
     const at::Tensor o = owned(pid, amp_master);
     if (o.grad().defined()) return in_param_shape(o.grad(), pid);
+    if (!o.is_cuda()) return in_param_shape(at::zeros_like(o.detach()), pid);   // a host tensor never reaches a kernel
     at::Tensor z = at::empty_like(o.detach());
     if (z.numel() > 0)
-      check(rg_fill_zero(z.data_ptr(), (int64_t)z.numel() * (int64_t)z.element_size(), z.is_cuda() ? z.get_device() : 0,
-                         z.is_cuda() ? current_stream(z.get_device()) : nullptr));
+      check(rg_fill_zero(z.data_ptr(), (int64_t)z.numel() * (int64_t)z.element_size(), z.get_device(), current_stream(z.get_device())));
     return in_param_shape(z, pid);
   }
   // doSyncParam + bcastParam (src/comp/ParamStorage.cpp:1079-1133) at one rank: the root's copy on the host

@@ -153,6 +153,7 @@ class _FusedBase(torch.optim.Optimizer):
         if ptrs != st.grad_ptrs:
             st.table.update_pointers(grads=ptrs, stream=stream_handle(st.device))
             st.grad_ptrs = ptrs
+            st.fed_by = None      # a feed's record of what it last pushed into this table is stale from here on
             # the full path's record of what the table points at must not outlive this re-pointing: a later
             # full step with the old addresses would otherwise find them "unchanged" and skip the update
             hit = self._tables.get(st.key)

@@ -254,6 +254,31 @@ def test_compiled_module_norm_clip_and_zero_match_the_python_registry(dtypes):
 
 
 @pytest.mark.gpu
+def test_compiled_module_does_not_keep_gradients_alive():
+    """The tables keep raw addresses; the tensors behind them are released as soon as the launch is queued, so that
+    ``zero_grad(set_to_none=True)`` gives the memory back before the next backward pass allocates new gradients."""
+    named = {f"layer.{i}.w": torch.nn.Parameter(torch.randn(1 << 20, device="cuda:0")) for i in range(4)}
+    _ranncgrad.reset_param_storage()
+    mod = _ranncgrad.RaNNCModule(False, False, False, True, False)
+    mod.init(named, False)
+    try:
+        torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated()
+        for call in (mod.calc_grad_norm, lambda: mod.clip_grad_norm(1.0), mod.zero_grad):
+            for p in named.values():
+                p.grad = torch.ones_like(p)
+            assert torch.cuda.memory_allocated() >= base + 4 * (4 << 20)
+            call()
+            for p in named.values():
+                p.grad = None
+            torch.cuda.synchronize()
+            assert torch.cuda.memory_allocated() == base, call
+    finally:
+        mod.undeploy()
+        _ranncgrad.reset_param_storage()
+
+
+@pytest.mark.gpu
 def test_compiled_module_zero_segments_and_amp_masters():
     """enable_zero: layouts, local segments and aligned buffers of the compiled class follow the oracle's closed
     forms at one rank; with amp masters registered the norm is taken over the masters' gradients."""
