@@ -37,6 +37,7 @@ struct rg_plan {
   int64_t n_chunks = 0;
   bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
   int64_t write_tile_elems = kWriteTileElems;
+  unsigned accumulate_lds = 0;   // unused dynamic LDS of rg_accumulate's pass (resident-block cap)
   int xcd_reduce = 64;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
   int xcd_write = 0;                 //   ... when every source sits on the line grid of its destination
   int xcd_write_offgrid = 256;       //   ... when some source does not (see fill_chunk_records)
@@ -213,7 +214,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->device = device;
   p->n_tensors = n;
   p->host_tensors.resize((size_t)n);
-  int64_t total = 0, bytes = 0;
+  int64_t total = 0, bytes = 0, same_width_bytes = 0, mixed_width_bytes = 0;
   int widest_src = 2, widest_any = 2;
   for (int i = 0; i < n; ++i) {
     const int ss = elem_size(src_dtype[i]), ds = elem_size(dst_dtype[i]);
@@ -238,7 +239,10 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
     }
     total += numel[i];
     bytes += numel[i] * (ss + ds);
+    (ss == ds ? same_width_bytes : mixed_width_bytes) += numel[i] * (ss + ds);
   }
+  // resident-block cap of rg_accumulate's pass (rg_internal.h), by what most of the plan's bytes look like
+  p->accumulate_lds = same_width_bytes >= mixed_width_bytes ? kAccSameWidthLdsBytes : kAccMixedWidthLdsBytes;
   p->total_numel = total;
   p->total_bytes = bytes;
   // The Infinity Cache holds 256 MiB: below that a second pass can still hit in cache.
@@ -668,6 +672,7 @@ RG_API int rg_accumulate(rg_plan* p, float scale, void* stream) {
   DeviceGuard guard(p->device);
   PassArgs a = pass_args(p, scale);
   split_for_write(p, a);
+  a.dynamic_lds = p->accumulate_lds;
   RG_HIP(launch_pass(kModeWrite | kModeAccumulate, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }

@@ -93,6 +93,15 @@ __host__ __device__ inline int head_elems(uintptr_t addr, unsigned align, unsign
 constexpr int64_t kChunkQuantum = 2048;    // chunk sizes are multiples of this many elements
 constexpr int64_t kMaxChunkElems = 1 << 20;
 constexpr unsigned kReducePassLdsBytes = 32768;   // dynamic LDS of the streaming read-only pass: 5 resident blocks per compute unit
+// rg_accumulate's pass reads more than it writes (source and old destination in, destination out) and, like the
+// read-only pass, runs faster with fewer blocks resident per compute unit (measured on MI355X, streaming sizes):
+// with 16 bytes loaded from each side per lane and step (both sides equally wide) ten blocks of 128 threads instead
+// of sixteen gain 2-5 %, with 8 + 16 bytes (a 16-bit side and an fp32 side) twelve blocks gain 3-4 %; BERT-large's
+// bf16 gradients into fp32: 79.6 -> 83.8 % of peak, the ResNet's fp32 into fp32: 79.3 -> 81.7 %.  The pass that also
+// sums (rg_unscale_accumulate) gains on flat same-width data but loses on the ResNet's many small tensors and is left
+// alone; plain writing passes lose from the first block taken away.
+constexpr unsigned kAccSameWidthLdsBytes = 16384;   // 10 resident blocks
+constexpr unsigned kAccMixedWidthLdsBytes = 13600;  // 12 resident blocks
 constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan
 
 // Pass selection for the chunk kernel.
@@ -139,6 +148,7 @@ struct PassArgs {
   int32_t only_if_clipped;       // with `result`: the whole launch does nothing unless result->clipped is set
   int32_t src_is_dst;            // read the destination instead of the record's source (in-place rescale)
   int32_t chunks_per_block;      // launch_gated_pass only: consecutive chunks one block walks through
+  uint32_t dynamic_lds;          // host side only: unused dynamic LDS that caps the resident blocks (0: the mode's default)
 };
 
 struct ReduceArgs {

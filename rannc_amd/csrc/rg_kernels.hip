@@ -630,6 +630,7 @@ void launch_mode(const PassArgs& a, bool streaming, hipStream_t stream) {
   // streaming read-only pass is fastest with 4-5 blocks of 256 threads per unit instead of the 8 that fit
   // (7.1 -> 7.4 TB/s on 2.5e9 fp16 elements); every writing pass wants all the blocks it can get.
   unsigned lds = (MODE == kModeReduce && streaming) ? kReducePassLdsBytes : 0u;
+  if ((MODE & kModeAccumulate) != 0 && streaming && a.dynamic_lds != 0) lds = a.dynamic_lds;
 #ifdef RG_TUNING_ENV   // experiment builds only
   if (const char* env = getenv((MODE & kModeWrite) ? "RG_LDS_WRITE" : "RG_LDS_REDUCE")) lds = (unsigned)atoi(env);
 #endif
