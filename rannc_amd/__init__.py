@@ -10,6 +10,7 @@ PyTorch fallback for it.
 """
 from __future__ import annotations
 
+import ctypes
 import logging
 
 import torch
@@ -221,7 +222,7 @@ class RaNNCModule(_pyrannc.RaNNCModule):
         if self.enable_apex_amp:
             self._setup_amp_params()
             stash = getattr(self.optimizer, "_amp_stash", None)
-            max_f = float(torch.tensor(max_grad_norm, dtype=torch.float32))      # crosses the binding as a C float
+            max_f = ctypes.c_float(float(max_grad_norm)).value      # crosses the binding as a C float
             if stash is not None and stash.pending_finish:
                 from .amp import can_step_from_model_grads, decide_clip, finish_unscale
                 if can_step_from_model_grads(self.optimizer):

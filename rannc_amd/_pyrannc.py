@@ -10,6 +10,7 @@ from __future__ import annotations
 
 from typing import Optional, Dict, Tuple
 
+import ctypes
 import torch
 
 from .dist_param_locator import DistributedParamLocator
@@ -207,7 +208,7 @@ class RaNNCModule:
         self._check()
         if self._n is not None:
             return self._n.clip_grad_norm(max_grad_norm)          # narrowed to a C float at the binding
-        _param_storage.clip_grad_norm(self.graph_id, float(torch.tensor(max_grad_norm, dtype=torch.float32)),
+        _param_storage.clip_grad_norm(self.graph_id, ctypes.c_float(float(max_grad_norm)).value,
                                       self._use_amp_master_params)
 
     def calc_grad_norm(self) -> float:

@@ -688,6 +688,9 @@ RG_API int rg_unscale_accumulate(rg_plan* p, float inv_scale, void* stream) {
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   PassArgs a = pass_args(p, inv_scale);
+  // Twelve resident blocks: what this kernel's register count (76) allows anyway, and what measures best for it.
+  // Said here so that the pass does not speed up or slow down with the compiler's register allocation.
+  a.dynamic_lds = kAccMixedWidthLdsBytes;
   const int rc2 = tiled_reduce_write(p, a, kModeReduce | kModeWrite | kModeAccumulate, s);
   p->sums_describe_dst = rc2 == RG_OK;
   return rc2;

@@ -98,8 +98,8 @@ constexpr unsigned kReducePassLdsBytes = 32768;   // dynamic LDS of the streamin
 // with 16 bytes loaded from each side per lane and step (both sides equally wide) ten blocks of 128 threads instead
 // of sixteen gain 2-5 %, with 8 + 16 bytes (a 16-bit side and an fp32 side) twelve blocks gain 3-4 %; BERT-large's
 // bf16 gradients into fp32: 79.6 -> 83.8 % of peak, the ResNet's fp32 into fp32: 79.3 -> 81.7 %.  The pass that also
-// sums (rg_unscale_accumulate) gains on flat same-width data but loses on the ResNet's many small tensors and is left
-// alone; plain writing passes lose from the first block taken away.
+// sums (rg_unscale_accumulate) holds twelve blocks by its register count already (ten gain on flat same-width data
+// but lose on the ResNet's many small tensors); plain writing passes lose from the first block taken away.
 constexpr unsigned kAccSameWidthLdsBytes = 16384;   // 10 resident blocks
 constexpr unsigned kAccMixedWidthLdsBytes = 13600;  // 12 resident blocks
 constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan

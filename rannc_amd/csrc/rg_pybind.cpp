@@ -362,6 +362,8 @@ PYBIND11_MODULE(_ranncgrad, m) {
   m.attr("STEP_IGNORE_OVERFLOW") = (int)RG_STEP_IGNORE_OVERFLOW;
   m.attr("STEP_EXPECT_NO_CLIP") = (int)RG_STEP_EXPECT_NO_CLIP;
   m.def("version", &rg_version);
+  m.def("current_stream", [](int device) { return reinterpret_cast<uintptr_t>(current_stream(device)); }, py::arg("device"),
+        "the hipStream_t PyTorch currently launches on for this device, as an integer (c10::hip::getCurrentHIPStream)");
   m.def("aligned_numel", [](int64_t numel, int elem_size, int split) {
     const int64_t r = rg_aligned_numel(numel, elem_size, split);
     if (r < 0) throw std::invalid_argument(rg_last_error());

@@ -402,3 +402,64 @@ def test_invalidate_tables_after_rehoming_a_parameter():
         ref.step()
         for i, (p, t) in enumerate(zip(params, twins)):
             assert_bits_equal(p.detach(), t.detach(), f"param {i} after step {step}")
+
+
+@pytest.mark.parametrize("fused_cls", [FusedAdam, FusedSGD])
+def test_step_hooks_grad_mode_and_schedulers_behave_as_with_torch_optim(fused_cls):
+    """The fused optimizers bring their own wrapper around ``step`` (torch's costs about 10 us per call); what torch's
+    does for a caller must still happen: registered and global step hooks run in torch's order and may replace the
+    arguments, gradient mode is off inside the step and back afterwards, a closure runs with it on, a learning-rate
+    scheduler counts the steps, and a recording profiler sees the ``Optimizer.step#...`` range."""
+    from torch.optim.optimizer import register_optimizer_step_post_hook, register_optimizer_step_pre_hook
+    p = torch.nn.Parameter(torch.ones(1000, device=DEV))
+    opt = fused_cls([p], lr=0.1)
+    sched = torch.optim.lr_scheduler.StepLR(opt, step_size=2, gamma=0.5)
+    calls = []
+    closure_modes = []
+
+    def closure():
+        closure_modes.append(torch.is_grad_enabled())
+        return torch.tensor(3.0)
+
+    def swap_in_closure(o, args, kwargs):
+        calls.append("pre")
+        return (args[0], closure), kwargs           # new positional arguments: (self, closure)
+
+    handles = [register_optimizer_step_pre_hook(lambda o, a, k: calls.append("global_pre")),
+               opt.register_step_pre_hook(swap_in_closure),
+               opt.register_step_post_hook(lambda o, a, k: calls.append(("post", len(a)))),
+               register_optimizer_step_post_hook(lambda o, a, k: calls.append("global_post"))]
+    try:
+        for step in range(3):
+            p.grad = torch.full_like(p, 0.5)
+            assert torch.is_grad_enabled()
+            out = opt.step()
+            assert torch.is_grad_enabled()
+            assert float(out) == 3.0                 # the closure the pre-hook put in was called
+            sched.step()
+        assert calls == ["global_pre", "pre", ("post", 2), "global_post"] * 3
+        assert closure_modes == [True] * 3
+        assert opt.param_groups[0]["lr"] == pytest.approx(0.05)      # halved once after two counted steps
+    finally:
+        for h in handles:
+            h.remove()
+    ref = torch.nn.Parameter(torch.ones(1000))
+    ref_opt = {FusedAdam: torch.optim.Adam, FusedSGD: torch.optim.SGD}[fused_cls]([ref], lr=0.1)
+    ref_sched = torch.optim.lr_scheduler.StepLR(ref_opt, step_size=2, gamma=0.5)
+    for step in range(3):
+        ref.grad = torch.full_like(ref, 0.5)
+        ref_opt.step()
+        ref_sched.step()
+    torch.testing.assert_close(p.detach().cpu(), ref.detach(), rtol=2e-6, atol=1e-7)
+    # a recording profiler still sees the range torch's wrapper would have opened
+    p.grad = torch.full_like(p, 0.5)
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CPU]) as prof:
+        opt.step()
+    assert any(e.key == f"Optimizer.step#{fused_cls.__name__}.step" for e in prof.key_averages())
+    # an exception inside the step must not leave gradient mode off
+    def failing_closure():
+        raise ValueError("from the closure")
+
+    with pytest.raises(ValueError, match="from the closure"):
+        opt.step(failing_closure)
+    assert torch.is_grad_enabled()

@@ -262,6 +262,8 @@ def test_compiled_module_does_not_keep_gradients_alive():
     mod = _ranncgrad.RaNNCModule(False, False, False, True, False)
     mod.init(named, False)
     try:
+        import gc
+        gc.collect()                      # what earlier tests left in reference cycles must not be freed in mid-test
         torch.cuda.synchronize()
         base = torch.cuda.memory_allocated()
         for call in (mod.calc_grad_norm, lambda: mod.clip_grad_norm(1.0), mod.zero_grad):
@@ -272,7 +274,7 @@ def test_compiled_module_does_not_keep_gradients_alive():
             for p in named.values():
                 p.grad = None
             torch.cuda.synchronize()
-            assert torch.cuda.memory_allocated() == base, call
+            assert torch.cuda.memory_allocated() <= base, call
     finally:
         mod.undeploy()
         _ranncgrad.reset_param_storage()
