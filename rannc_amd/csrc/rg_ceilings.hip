@@ -15,11 +15,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ f32x4 as_f32x4(u32x4 v) { return __builtin_bit_cast(f32x4, v); }
 __device__ __forceinline__ u32x4 as_u32x4(f32x4 v) { return __builtin_bit_cast(u32x4, v); }
 
-// Streaming store with the cache policy of the passes that write one stream per launch.
-__device__ __forceinline__ void st16_stream(char* p, u32x4 v) {
-  RG_GLOBAL u32x4* g = (RG_GLOBAL u32x4*)p;
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(g), "v"(v) : "memory");   // two wait states: the compiler does not know this is a 128-bit store whose data registers must not be overwritten yet
-}
+// Streaming store as the passes that write one stream per launch issue it (buffer store, nt sc1).
+__device__ __forceinline__ void st16_stream(char* p, u32x4 v) { st16_aux<2 | 16>(p, v); }
 
 // Read only: the read-only pass's shape.  256 threads, eight 16-byte nontemporal loads in flight per
 // lane (32 KiB per block), launched with the same unused dynamic LDS that caps the resident blocks.

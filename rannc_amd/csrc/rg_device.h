@@ -48,14 +48,41 @@ template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
 }
 // Stores: the pointer type promises element alignment only (what the peel guarantees beyond
 // that is a performance matter, not a correctness one).
-// Streaming (NT) stores come in two forms.  The default is the compiler's nontemporal store
-// (`nt`).  A translation unit that defines RG_STREAM_STORE_BITS before including this header
-// gets its streaming stores issued with exactly those cache-policy bits instead: measured on
-// MI355X, "sc1 nt" (agent-scope write-through, streaming) is 1.5-3 % faster than plain `nt`
-// for the passes that write one stream per launch and slower for the optimizer step's three.
+//
+// Streaming (NT) stores come in three forms.  The default is the compiler's nontemporal store (`nt`).  A
+// translation unit that defines RG_STREAM_STORE_AUX before including this header gets them issued as raw buffer
+// stores with those cache-policy bits (1 = sc0, 2 = nt, 16 = sc1): measured on MI355X, "sc1 nt" (agent-scope
+// write-through, streaming) is 1.5-3 % faster than plain `nt` for the passes that write one stream per launch and
+// slower for the optimizer step's three.  Buffer instructions because they take the bits as an operand and - unlike
+// a global store spelled out in an asm statement, which RG_STREAM_STORE_BITS still offers for comparison - are
+// known to the compiler's wait-count bookkeeping: with an invisible store in flight the compiler believes the load
+// it waits for is the only outstanding operation and drains the whole counter (vmcnt(0)), store included, where
+// vmcnt(1) would do.  That over-wait, not the store, was what a pass paid for whenever it had work left after its
+// last store (the pass that sums while it writes: 4-5 %).
+//
+// The descriptor's base is the address of the wavefront's first active lane, the lane's distance from it the
+// offset: lanes ascend in address in every kernel of this library.
 #ifndef RG_NT_STORES
 #define RG_NT_STORES 1
 #endif
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_window(char* p, uint32_t& off) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  const uint64_t base = ((uint64_t)hi << 32) | lo;
+  off = (uint32_t)(a - base);
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, -1, 0x00020000);   // raw, unbounded
+}
+template <int AUX> __device__ __forceinline__ void st16_aux(char* p, u32x4 v) {
+  uint32_t off;
+  const __amdgpu_buffer_rsrc_t r = wave_window(p, off);
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, AUX);
+}
+template <int AUX> __device__ __forceinline__ void st8_aux(char* p, u32x2 v) {
+  uint32_t off;
+  const __amdgpu_buffer_rsrc_t r = wave_window(p, off);
+  __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, AUX);
+}
 // gfx940-family hazard: a VALU instruction that overwrites the data registers of a store of more than 64 bits
 // within two wait states of it changes what is stored.  The compiler spaces its own stores accordingly, but it
 // does not know that an asm statement is a store, so every 128-bit store issued through asm brings its own two
@@ -63,7 +90,12 @@ template <bool NT> __device__ __forceinline__ u32x2 ld8_a2(const char* p) {
 #define RG_STORE_HAZARD_NOP "\n\ts_nop 1"
 template <bool NT> __device__ __forceinline__ void st16(char* p, u32x4 v) {
   RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
-#ifdef RG_STREAM_STORE_BITS
+#if defined(RG_STREAM_STORE_AUX)
+  if (NT) {
+    st16_aux<RG_STREAM_STORE_AUX>(p, v);
+    return;
+  }
+#elif defined(RG_STREAM_STORE_BITS)
   if (NT) {
     asm volatile("global_store_dwordx4 %0, %1, off " RG_STREAM_STORE_BITS RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
     return;
@@ -74,7 +106,12 @@ template <bool NT> __device__ __forceinline__ void st16(char* p, u32x4 v) {
 }
 template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
   RG_GLOBAL u32x2_a2* g = (RG_GLOBAL u32x2_a2*)p;
-#ifdef RG_STREAM_STORE_BITS
+#if defined(RG_STREAM_STORE_AUX)
+  if (NT) {
+    st8_aux<RG_STREAM_STORE_AUX>(p, v);
+    return;
+  }
+#elif defined(RG_STREAM_STORE_BITS)
   if (NT) {
     asm volatile("global_store_dwordx2 %0, %1, off " RG_STREAM_STORE_BITS : : "v"(g), "v"(v));
     return;
@@ -82,33 +119,6 @@ template <bool NT> __device__ __forceinline__ void st8(char* p, u32x2 v) {
 #endif
   if (NT && RG_NT_STORES) __builtin_nontemporal_store(v, g);
   else *g = v;
-}
-
-// Stores whose order in the instruction stream is fixed (volatile asm statements keep their relative order):
-// st16_ordered is a plain 16-byte store, st16_last / st8_last are the stores above issued after it.
-__device__ __forceinline__ void st16_ordered(char* p, u32x4 v) {
-  RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
-  asm volatile("global_store_dwordx4 %0, %1, off" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
-}
-template <bool NT> __device__ __forceinline__ void st16_last(char* p, u32x4 v) {
-  RG_GLOBAL u32x4_a2* g = (RG_GLOBAL u32x4_a2*)p;
-#ifdef RG_STREAM_STORE_BITS
-  if (NT) asm volatile("global_store_dwordx4 %0, %1, off " RG_STREAM_STORE_BITS RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
-  else asm volatile("global_store_dwordx4 %0, %1, off" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
-#else
-  if (NT) asm volatile("global_store_dwordx4 %0, %1, off nt" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
-  else asm volatile("global_store_dwordx4 %0, %1, off" RG_STORE_HAZARD_NOP : : "v"(g), "v"(v));
-#endif
-}
-template <bool NT> __device__ __forceinline__ void st8_last(char* p, u32x2 v) {
-  RG_GLOBAL u32x2_a2* g = (RG_GLOBAL u32x2_a2*)p;
-#ifdef RG_STREAM_STORE_BITS
-  if (NT) asm volatile("global_store_dwordx2 %0, %1, off " RG_STREAM_STORE_BITS : : "v"(g), "v"(v));
-  else asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(g), "v"(v));
-#else
-  if (NT) asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(g), "v"(v));
-  else asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(g), "v"(v));
-#endif
 }
 
 template <int DT, int E, bool NT> struct Mem;
@@ -206,24 +216,32 @@ template <> __device__ __forceinline__ float round_dst<RG_BF16>(float v) {
   return bf16_bits_to_f32(f32_to_bf16_bits(v));
 }
 
+// One element at a time (unaligned heads, ragged tails, the re-scan after a non-finite sum).  Through pointers of
+// the global address space, like the vector accesses: a generic pointer compiles to FLAT instructions, which count
+// on two of the wave's counters at once, and the compiler then waits for both to drain (vmcnt(0) lgkmcnt(0)) before
+// it reuses one of their registers - a wait that also covers every vector store still in flight.
 template <int DT> __device__ __forceinline__ void store1(char* p, float v) {
-  *reinterpret_cast<float*>(p) = v;
+  *(RG_GLOBAL float*)p = v;
 }
 template <> __device__ __forceinline__ void store1<RG_F16>(char* p, float v) {
-  *reinterpret_cast<_Float16*>(p) = f32_to_f16(v);
+  *(RG_GLOBAL _Float16*)p = f32_to_f16(v);
 }
 template <> __device__ __forceinline__ void store1<RG_BF16>(char* p, float v) {
-  *reinterpret_cast<unsigned short*>(p) = (unsigned short)f32_to_bf16_bits(v);
+  *(RG_GLOBAL unsigned short*)p = (unsigned short)f32_to_bf16_bits(v);
 }
+__device__ __forceinline__ uint32_t load_u32(const char* p) { return *(const RG_GLOBAL uint32_t*)p; }
+__device__ __forceinline__ uint32_t load_u16(const char* p) { return (uint32_t)*(const RG_GLOBAL unsigned short*)p; }
+__device__ __forceinline__ void store_u32(char* p, uint32_t v) { *(RG_GLOBAL uint32_t*)p = v; }
+__device__ __forceinline__ void store_u16(char* p, uint32_t v) { *(RG_GLOBAL unsigned short*)p = (unsigned short)v; }
 
 template <int DT> __device__ __forceinline__ bool nonfinite_at(const char* p) {
-  return (*reinterpret_cast<const uint32_t*>(p) & 0x7f800000u) == 0x7f800000u;
+  return (load_u32(p) & 0x7f800000u) == 0x7f800000u;
 }
 template <> __device__ __forceinline__ bool nonfinite_at<RG_F16>(const char* p) {
-  return (*reinterpret_cast<const unsigned short*>(p) & 0x7c00u) == 0x7c00u;
+  return (load_u16(p) & 0x7c00u) == 0x7c00u;
 }
 template <> __device__ __forceinline__ bool nonfinite_at<RG_BF16>(const char* p) {
-  return (*reinterpret_cast<const unsigned short*>(p) & 0x7f80u) == 0x7f80u;
+  return (load_u16(p) & 0x7f80u) == 0x7f80u;
 }
 
 // Sum of one double per lane over the 64-lane wavefront, the same value returned to every
@@ -249,22 +267,6 @@ __device__ __forceinline__ double wave_total(double x) {
   x += dpp_row_shr<4>(x);
   x += dpp_row_shr<8>(x);
   return (read_lane(x, 15) + read_lane(x, 31)) + (read_lane(x, 47) + read_lane(x, 63));
-}
-
-// Sum of one float per lane over the wavefront in six DPP additions (two butterflies inside each quad, two row
-// shifts, two row broadcasts: ((r3 + r2) + (r1 + r0)) of the row sums ends up in lane 63), returned to every lane.
-// All 64 lanes must be active.
-template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_f32(float x) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, ROW_MASK, 0xf, false));
-}
-__device__ __forceinline__ float wave_total_f32(float x) {
-  x += dpp_f32<0xb1, 0xf>(x);    // quad_perm:[1,0,3,2]
-  x += dpp_f32<0x4e, 0xf>(x);    // quad_perm:[2,3,0,1]
-  x += dpp_f32<0x114, 0xf>(x);   // row_shr:4
-  x += dpp_f32<0x118, 0xf>(x);   // row_shr:8
-  x += dpp_f32<0x142, 0xa>(x);   // row_bcast:15 into rows 1 and 3
-  x += dpp_f32<0x143, 0xc>(x);   // row_bcast:31 into rows 2 and 3
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
 }
 
 }  // namespace

@@ -23,12 +23,23 @@
 #include <cstdlib>
 #include <type_traits>
 
-// the passes of this file write one stream per launch: see the note on streaming stores in rg_device.h
-#if !defined(RG_STREAM_STORE_BITS) && !defined(RG_STREAM_STORE_COMPILER_NT)
-#define RG_STREAM_STORE_BITS "sc1 nt"
+// the passes of this file write one stream per launch: see the notes on streaming stores in rg_device.h
+#if !defined(RG_STREAM_STORE_AUX) && !defined(RG_STREAM_STORE_BITS) && !defined(RG_STREAM_STORE_COMPILER_NT)
+#define RG_STREAM_STORE_AUX (2 | 16)   // nt sc1
 #endif
 #include "rg_device.h"
 #include "rg_internal.h"
+
+// steps of a writing pass whose loads are issued together (see process_chunk)
+#ifndef RG_WRITE_STEPS_IN_FLIGHT
+#define RG_WRITE_STEPS_IN_FLIGHT 1
+#endif
+#ifndef RG_SUM_WRITE_STEPS_IN_FLIGHT
+#define RG_SUM_WRITE_STEPS_IN_FLIGHT 2
+#endif
+#ifndef RG_ACC_STEPS_IN_FLIGHT
+#define RG_ACC_STEPS_IN_FLIGHT 1
+#endif
 
 namespace rg {
 namespace {
@@ -40,29 +51,9 @@ template <int MODE> struct PassThreads { static constexpr int value = (MODE & kM
 // coef is 1 when nothing is clipped: v * 1 is v bit for bit, so no branch is needed.
 // The two multiplies are never fused or reassociated (the file is built with
 // -ffp-contract=off), so the result matches `x.float() * inv_scale` then `mul_(coef)`.
-// A vector store that process_chunk holds back for its caller (bytes == 0: none).
-struct PendingStore {
-  u32x4 v;
-  char* p;
-  int bytes;
-};
-
-#ifndef RG_DEFER_LAST_STORE
-#define RG_DEFER_LAST_STORE 1
-#endif
-// A pass that sums while it writes ends every wavefront with a store that depends on everything before it: the
-// record of its partial sum.  Measured on MI355X, that trailing store costs such a pass 4-5 % whatever its size,
-// cache policy or address (a record stored in mid-life, or none at all, costs nothing: the time goes into the end
-// of blocks that live under 4 us).  With fp32 sources most of it comes back when the last vector store is held
-// back until the record has been issued - the caller reduces, stores the record, then the held vector - (+5-7 %
-// for fp32 -> fp32 / bf16 / fp16); with 16-bit sources the same reordering loses 2 %, so they keep the plain order.
-template <int S, int MODE> struct DefersLastStore {
-  static constexpr bool value = RG_DEFER_LAST_STORE && S == RG_F32 && (MODE & kModeReduce) != 0 && (MODE & kModeWrite) != 0;
-};
-
 template <int S, int D, int MODE, bool NT, int T = PassThreads<MODE>::value, bool HEAD = true>
 __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len, float scale, float coef,
-                                              bool raw_copy, float (&acc)[8], PendingStore& pending) {
+                                              bool raw_copy, float (&acc)[8]) {
   constexpr int SS = ElemSize<S>::value;
   constexpr int DS = ElemSize<D>::value;
   constexpr bool kWrite = (MODE & kModeWrite) != 0;
@@ -70,8 +61,12 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   constexpr bool kAcc = (MODE & kModeAccumulate) != 0;   // dst = round_dst(float(dst) + x * scale)
   constexpr int E = (SS == 4 || (kWrite && DS == 4)) ? 4 : 8;   // elements per lane per instruction
   // a read-only pass keeps 128 bytes of source in flight per lane (eight 16-byte loads) whatever the element size
-  constexpr int kPerThread = kWrite ? kWriteElemsPerThread : kReduceElemsPerThread * (4 / SS);
-  constexpr int U = kPerThread >= E ? kPerThread / E : 1;      // instructions in flight per lane
+  // A writing pass moves one vector per lane and step.  The pass that also sums issues the loads of both its steps
+  // before the first store (measured with stores the compiler can account for: +1.5-3 points on every workload,
+  // where the plain write pass loses 0.5-1.5 with 16-bit sources and the accumulating passes lose 1-2).
+  constexpr int kSteps = kAcc ? RG_ACC_STEPS_IN_FLIGHT : ((kReduce && kWrite) ? RG_SUM_WRITE_STEPS_IN_FLIGHT : RG_WRITE_STEPS_IN_FLIGHT);
+  constexpr int kPerThread = kReduceElemsPerThread * (4 / SS);   // read-only pass
+  constexpr int U = kWrite ? kSteps * (kWriteElemsPerThread / 4) : (kPerThread >= E ? kPerThread / E : 1);   // instructions in flight per lane
   constexpr int AS = kWrite ? DS : SS;
   constexpr unsigned kPeel = kWrite ? kWriteAlignBytes : kAlignBytes;
   const uintptr_t a = kWrite ? reinterpret_cast<uintptr_t>(dp) : reinterpret_cast<uintptr_t>(sp);
@@ -82,19 +77,19 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   const int tail0 = head + nbody;
   const int tid = threadIdx.x;
 
-  // Unaligned head (read-only pass: < 128 bytes) and ragged tail (< E elements): one element per thread.
-  // The element is loaded here, before the vector loop, and converted and stored after it,
-  // so its memory latency overlaps the vector loads instead of preceding them.
+  // Unaligned head (read-only pass: < 128 bytes) and ragged tail (< E elements): one element per thread, after the
+  // vector loop (a load issued up here, to overlap its latency with the vector loads, leaves the compiler with a
+  // register it believes in flight on the path around that loop, and the wait it then places behind the loop - for
+  // every block, with or without scalar elements - also waits for the vector stores: see the end of this function).
   const int nscalar = head + (len - tail0);
   auto scalar_index = [&](int k) { return k < head ? k : tail0 + (k - head); };
   auto scalar_load = [&](int i) -> uint32_t {
-    return SS == 4 ? *reinterpret_cast<const uint32_t*>(sp + (size_t)i * 4)
-                   : (uint32_t)*reinterpret_cast<const unsigned short*>(sp + (size_t)i * 2);
+    return SS == 4 ? load_u32(sp + (size_t)i * 4) : load_u16(sp + (size_t)i * 2);
   };
   auto scalar_finish = [&](uint32_t raw, int i) {
     if (S == D && raw_copy) {
-      if (SS == 4) *reinterpret_cast<uint32_t*>(dp + (size_t)i * 4) = raw;
-      else *reinterpret_cast<unsigned short*>(dp + (size_t)i * 2) = (unsigned short)raw;
+      if (SS == 4) store_u32(dp + (size_t)i * 4, raw);
+      else store_u16(dp + (size_t)i * 2, raw);
     } else {
       float x;
       if (S == RG_F32) x = __uint_as_float(raw);
@@ -103,9 +98,9 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
       float t = x * scale;
       if (kAcc) {
         float old;
-        if (D == RG_F32) old = *reinterpret_cast<const float*>(dp + (size_t)i * 4);
-        else if (D == RG_F16) old = f16_to_f32(*reinterpret_cast<const _Float16*>(dp + (size_t)i * 2));
-        else old = bf16_bits_to_f32(*reinterpret_cast<const unsigned short*>(dp + (size_t)i * 2));
+        if (D == RG_F32) old = __uint_as_float(load_u32(dp + (size_t)i * 4));
+        else if (D == RG_F16) old = f16_to_f32(__builtin_bit_cast(_Float16, (unsigned short)load_u16(dp + (size_t)i * 2)));
+        else old = bf16_bits_to_f32(load_u16(dp + (size_t)i * 2));
         t = opaque(t) + old;
       }
       const float v = round_dst<D>(t);
@@ -113,10 +108,6 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
       if (kWrite) store1<D>(dp + (size_t)i * DS, v * coef);
     }
   };
-  const bool has_scalar = tid < nscalar;
-  const int scalar_i = has_scalar ? scalar_index(tid) : 0;
-  uint32_t scalar_raw = 0;
-  if (has_scalar) scalar_raw = scalar_load(scalar_i);
 
   const char* sb = sp + (size_t)head * SS;
   char* db = dp + (size_t)head * DS;
@@ -127,8 +118,7 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   // previous destination values, only when accumulating (the type does not exist otherwise)
   struct Nothing {};
   using Old = std::conditional_t<kAcc, Raw<kAcc ? D : S, E>, Nothing>;
-  constexpr bool kDefer = DefersLastStore<S, MODE>::value;
-  auto consume = [&](const Raw<S, E>& in, const Old* old, int e, bool valid, bool hold) {
+  auto consume = [&](const Raw<S, E>& in, const Old* old, int e, bool valid) {
     bool copied = false;
     if constexpr (S == D && kWrite) {
       if (raw_copy) {
@@ -153,21 +143,7 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
         if (kWrite) f[j] = round_dst<D>(v * coef);
       }
       if constexpr (kWrite) {
-        if constexpr (kDefer) {
-          if (hold) {
-            if (valid) {
-              const Raw<D, E> out = Codec<D, E>::pack(f);
-              if constexpr (sizeof(out.v) == 16) pending.v = out.v;
-              else pending.v = u32x4{out.v[0], out.v[1], 0u, 0u};
-              pending.p = db + (size_t)e * DS;
-              pending.bytes = (int)sizeof(out.v);
-            }
-          } else if (valid) {
-            Mem<D, E, NT>::store(db + (size_t)e * DS, Codec<D, E>::pack(f));
-          }
-        } else {
-          if (valid) Mem<D, E, NT>::store(db + (size_t)e * DS, Codec<D, E>::pack(f));
-        }
+        if (valid) Mem<D, E, NT>::store(db + (size_t)e * DS, Codec<D, E>::pack(f));
       }
     }
   };
@@ -182,10 +158,8 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
 #pragma unroll
       for (int u = 0; u < U; ++u) old[u] = Mem<D, E, NT>::load(db + (size_t)(base + (u * T + tid) * E) * DS);
     }
-    // the last vector store of the chunk is the one held back (only its final instruction: u == U - 1)
-    const bool final_iter = kDefer && base + kIter == nbody;
 #pragma unroll
-    for (int u = 0; u < U; ++u) consume(in[u], &old[kAcc ? u : 0], base + (u * T + tid) * E, true, final_iter && u == U - 1);
+    for (int u = 0; u < U; ++u) consume(in[u], &old[kAcc ? u : 0], base + (u * T + tid) * E, true);
   }
   if (base < nbody) {
     // Last, partial iteration: lanes past the end re-read the final vector (an address that
@@ -201,14 +175,25 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int e = base + (u * T + tid) * E;
-      consume(in[u], &old[kAcc ? u : 0], e, e < nbody, kDefer && u == U - 1);
+      consume(in[u], &old[kAcc ? u : 0], e, e < nbody);
     }
   }
 
-  if (has_scalar) scalar_finish(scalar_raw, scalar_i);
-  for (int k = tid + T; k < nscalar; k += T) {
-    const int i = scalar_index(k);
-    scalar_finish(scalar_load(i), i);
+  // Block-uniform: most tiles have neither head nor tail.  The scalar stores in here are the only memory operations
+  // the compiler knows to be in flight (the streaming vector stores are asm statements), and it waits for them -
+  // with vmcnt(0), which covers those vector stores as well - before the first later instruction that reuses one of
+  // their registers.  Left to the compiler that wait lands behind the join, in the path of every wavefront: a pass
+  // that goes on to reduce and store a record then sits there until its last vector store has been acknowledged,
+  // one more trip to memory in a block that lives for two (measured: 4-5 % of the pass).  Waiting inside the
+  // branch keeps the common path free of it.
+  if (nscalar > 0) {
+    for (int k = tid; k < nscalar; k += T) {
+      const int i = scalar_index(k);
+      scalar_finish(scalar_load(i), i);
+    }
+#ifndef RG_NO_TAIL_WAIT
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0), expcnt untouched
+#endif
   }
 }
 
@@ -224,7 +209,7 @@ __device__ __forceinline__ void zero_range(char* p, int nbytes) {
   const int nscalar = (head + (nbytes - tail0)) / 2;
   for (int k = tid; k < nscalar; k += T) {
     const int off = k < head / 2 ? k * 2 : tail0 + (k - head / 2) * 2;
-    *reinterpret_cast<unsigned short*>(p + off) = 0;
+    store_u16(p + off, 0u);
   }
   const u32x4 z = {0u, 0u, 0u, 0u};
   for (int v = tid; v < nvec; v += T) st16<NT>(p + head + (size_t)v * 16, z);
@@ -296,14 +281,13 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
   const bool raw_copy = (MODE == kModeWrite) && a.result == nullptr && a.scale_dev == nullptr && a.scale == 1.0f;   // never when accumulating
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  PendingStore pending{u32x4{0u, 0u, 0u, 0u}, nullptr, 0};
   if (sp == nullptr || a.zero_fill) {
     if constexpr ((MODE & kModeAccumulate) != 0) {
       // Nothing to add: the destination keeps its values, which still count towards the norm.
       if constexpr ((MODE & kModeReduce) != 0) {
-        if (dst_kind == RG_F32) process_chunk<RG_F32, RG_F32, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc, pending);
-        else if (dst_kind == RG_F16) process_chunk<RG_F16, RG_F16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc, pending);
-        else process_chunk<RG_BF16, RG_BF16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc, pending);
+        if (dst_kind == RG_F32) process_chunk<RG_F32, RG_F32, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
+        else if (dst_kind == RG_F16) process_chunk<RG_F16, RG_F16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
+        else process_chunk<RG_BF16, RG_BF16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
       }
     } else if (MODE & kModeWrite) {
       zero_range<NT, T, PEEL>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
@@ -316,8 +300,8 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
     const bool has_head = ((MODE & kModeWrite) == 0 || PEEL) && (peeled & (peel - 1)) != 0;
 #define RG_PAIR(S, D)                                                                         \
   case S * 3 + D:                                                                             \
-    if (has_head) process_chunk<S, D, MODE, NT, T, true>(sp, dp, len, scale, coef, raw_copy, acc, pending);  \
-    else process_chunk<S, D, MODE, NT, T, false>(sp, dp, len, scale, coef, raw_copy, acc, pending);  \
+    if (has_head) process_chunk<S, D, MODE, NT, T, true>(sp, dp, len, scale, coef, raw_copy, acc);  \
+    else process_chunk<S, D, MODE, NT, T, false>(sp, dp, len, scale, coef, raw_copy, acc);  \
     break;
     switch (src_kind * 3 + dst_kind) {
       RG_PAIR(RG_F32, RG_F32)
@@ -329,8 +313,8 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
       RG_PAIR(RG_BF16, RG_F32)
       RG_PAIR(RG_BF16, RG_F16)
       default:
-        if (has_head) process_chunk<RG_BF16, RG_BF16, MODE, NT, T, true>(sp, dp, len, scale, coef, raw_copy, acc, pending);
-        else process_chunk<RG_BF16, RG_BF16, MODE, NT, T, false>(sp, dp, len, scale, coef, raw_copy, acc, pending);
+        if (has_head) process_chunk<RG_BF16, RG_BF16, MODE, NT, T, true>(sp, dp, len, scale, coef, raw_copy, acc);
+        else process_chunk<RG_BF16, RG_BF16, MODE, NT, T, false>(sp, dp, len, scale, coef, raw_copy, acc);
         break;
     }
 #undef RG_PAIR
@@ -358,25 +342,11 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
         return __any(mine) ? 1 : 0;
       };
       Partial* const slot = &a.partials[slot_id * kSlots + (threadIdx.x >> 6)];
-      if (RG_DEFER_LAST_STORE && src_kind == RG_F32 && sp != nullptr) {
-        // process_chunk held the last vector store back, and that store now waits for the record.  The 8 elements
-        // of a lane and the 64 lanes are therefore added in fp32 (six DPP additions in a fixed order): 512 squares
-        // summed as a tree are within a few 1e-8 of their exact sum, and everything after the record is double.
-        const float lane_sum = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
-        const float total = wave_total_f32(lane_sum);
-        const int bad = !(fabsf(total) <= 3.40282346638528859812e38f) ? rescan() : 0;
-        // the record, then the held vector: both through volatile asm, which keeps their order
-        const Partial rec{(double)total, bad, 0};
-        if ((threadIdx.x & 63) == 0) st16_ordered(reinterpret_cast<char*>(slot), __builtin_bit_cast(u32x4, rec));
-        if (pending.bytes == 16) st16_last<NT>(pending.p, pending.v);
-        else if (pending.bytes == 8) st8_last<NT>(pending.p, u32x2{pending.v[0], pending.v[1]});
-      } else {
-        double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
-                   (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
-        s = wave_total(s);
-        const int bad = !(fabs(s) <= 1.79769313486231570e308) ? rescan() : 0;
-        if ((threadIdx.x & 63) == 0) *slot = Partial{s, bad, 0};
-      }
+      double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
+                 (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
+      s = wave_total(s);
+      const int bad = !(fabs(s) <= 1.79769313486231570e308) ? rescan() : 0;
+      if ((threadIdx.x & 63) == 0) *slot = Partial{s, bad, 0};
     } else {
       // One partial per block: the 8 sums of the thread, the 64 lanes of the wavefront by DPP row scans, the
       // wavefronts through LDS in index order.  Everything past the per-thread fp32 sums is double.

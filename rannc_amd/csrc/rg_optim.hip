@@ -110,12 +110,12 @@ __device__ __forceinline__ void update_one(float& p, float g, float& s1, float& 
   }
 }
 
-template <int DT> __device__ __forceinline__ float load1(const char* p) { return *reinterpret_cast<const float*>(p); }
+template <int DT> __device__ __forceinline__ float load1(const char* p) { return __uint_as_float(load_u32(p)); }
 template <> __device__ __forceinline__ float load1<RG_F16>(const char* p) {
-  return f16_to_f32(*reinterpret_cast<const _Float16*>(p));
+  return f16_to_f32(__builtin_bit_cast(_Float16, (unsigned short)load_u16(p)));
 }
 template <> __device__ __forceinline__ float load1<RG_BF16>(const char* p) {
-  return bf16_bits_to_f32(*reinterpret_cast<const unsigned short*>(p));
+  return bf16_bits_to_f32(load_u16(p));
 }
 
 // One tile of one chunk.  G: gradient dtype; C: model-copy dtype, or -1 for none.
@@ -147,14 +147,14 @@ __device__ __forceinline__ void optim_tile(const OptChunkRec& r, int start, int 
   const int nscalar = head + (len - tail0);
   for (int k = tid; k < nscalar; k += T) {
     const int i = k < head ? k : tail0 + (k - head);
-    float p = *reinterpret_cast<const float*>(pp + (size_t)i * 4);
+    float p = __uint_as_float(load_u32(pp + (size_t)i * 4));
     const float g = load1<G>(gp + (size_t)i * GS);
-    float s1 = use_s1 ? *reinterpret_cast<const float*>(s1p + (size_t)i * 4) : 0.0f;
-    float s2 = ALGO == kAdam ? *reinterpret_cast<const float*>(s2p + (size_t)i * 4) : 0.0f;
+    float s1 = use_s1 ? __uint_as_float(load_u32(s1p + (size_t)i * 4)) : 0.0f;
+    float s2 = ALGO == kAdam ? __uint_as_float(load_u32(s2p + (size_t)i * 4)) : 0.0f;
     update_one<ALGO>(p, g, s1, s2, c, coef);
-    *reinterpret_cast<float*>(pp + (size_t)i * 4) = p;
-    if (use_s1) *reinterpret_cast<float*>(s1p + (size_t)i * 4) = s1;
-    if (ALGO == kAdam) *reinterpret_cast<float*>(s2p + (size_t)i * 4) = s2;
+    store_u32(pp + (size_t)i * 4, __float_as_uint(p));
+    if (use_s1) store_u32(s1p + (size_t)i * 4, __float_as_uint(s1));
+    if (ALGO == kAdam) store_u32(s2p + (size_t)i * 4, __float_as_uint(s2));
     if (kCopy) store1<CD>(cp + (size_t)i * CS, p);
   }
 

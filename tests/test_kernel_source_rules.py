@@ -32,4 +32,4 @@ def test_every_128_bit_asm_store_waits_two_states():
             for name, value in macros.items():
                 template = template.replace(name, '"' + value + '"')
             assert "s_nop 1" in template, f"{os.path.basename(path)}: 128-bit asm store without its wait states: {stmt.strip()[:120]}"
-    assert seen >= 4, "expected to find the library's asm stores"
+    assert seen >= 1, "expected to find the asm store the header keeps for comparison builds"
