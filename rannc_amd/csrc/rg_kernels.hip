@@ -34,6 +34,9 @@
 #ifndef RG_WRITE_STEPS_IN_FLIGHT
 #define RG_WRITE_STEPS_IN_FLIGHT 1
 #endif
+#ifndef RG_WRITE_STEPS_IN_FLIGHT_F32
+#define RG_WRITE_STEPS_IN_FLIGHT_F32 1
+#endif
 #ifndef RG_SUM_WRITE_STEPS_IN_FLIGHT
 #define RG_SUM_WRITE_STEPS_IN_FLIGHT 2
 #endif
@@ -64,7 +67,7 @@ __device__ __forceinline__ void process_chunk(const char* sp, char* dp, int len,
   // A writing pass moves one vector per lane and step.  The pass that also sums issues the loads of both its steps
   // before the first store (measured with stores the compiler can account for: +1.5-3 points on every workload,
   // where the plain write pass loses 0.5-1.5 with 16-bit sources and the accumulating passes lose 1-2).
-  constexpr int kSteps = kAcc ? RG_ACC_STEPS_IN_FLIGHT : ((kReduce && kWrite) ? RG_SUM_WRITE_STEPS_IN_FLIGHT : RG_WRITE_STEPS_IN_FLIGHT);
+  constexpr int kSteps = kAcc ? RG_ACC_STEPS_IN_FLIGHT : ((kReduce && kWrite) ? RG_SUM_WRITE_STEPS_IN_FLIGHT : (SS == 4 ? RG_WRITE_STEPS_IN_FLIGHT_F32 : RG_WRITE_STEPS_IN_FLIGHT));
   constexpr int kPerThread = kReduceElemsPerThread * (4 / SS);   // read-only pass
   constexpr int U = kWrite ? kSteps * (kWriteElemsPerThread / 4) : (kPerThread >= E ? kPerThread / E : 1);   // instructions in flight per lane
   constexpr int AS = kWrite ? DS : SS;
