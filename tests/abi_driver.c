@@ -174,6 +174,54 @@ int main(void) {
     CHECK_HIP(hipMemcpy(d_src + 2 * 77777, &h_src[77777], 2, hipMemcpyHostToDevice));
   }
 
+  /* ---- the loss scale on the device: the unscale reads 1/scale from the scaler's state, the schedule follows the
+   *      result block - a clean step counts (window 2: the second one doubles the scale), an overflow halves it */
+  {
+    rg_scaler_state init, st, *d_state = NULL;
+    const rg_step_result* d_result = NULL;
+    memset(&init, 0, sizeof(init));
+    init.loss_scale = scale; /* 64: the gradients above carry exactly this scale */
+    init.max_loss_scale = 256.0f;
+    init.scale_window = 2;
+    init.scale_factor = 2.0f;
+    CHECK_HIP(hipMalloc((void**)&d_state, sizeof(rg_scaler_state)));
+    CHECK_RG(rg_scaler_init(d_state, &init, device, NULL));
+    CHECK_RG(rg_result_device_ptr(plan, &d_result));
+    CHECK_HIP(hipMemset(d_dst, 0x22, (size_t)total * 4));
+    CHECK_RG(rg_step_begin_scaled(plan, &d_state->inv_scale, NULL));
+    CHECK_RG(rg_step_finish(plan, max_norm, RG_STEP_DEFAULT, NULL));
+    CHECK_RG(rg_scaler_update(d_state, d_result, RG_SCALER_DYNAMIC | RG_SCALER_TRUNCATE, device, NULL));
+    CHECK_RG(rg_read_result(plan, &res, NULL));
+    EXPECT(res.overflow == 0 && res.clipped == 1 && fabs(res.norm - norm) <= 1e-6 * norm);
+    CHECK_HIP(hipMemcpy(h_got, d_dst, (size_t)total * 4, hipMemcpyDeviceToHost));
+    EXPECT(same_bits(h_got, h_want, total)); /* the same bits as with the scale passed by value */
+    CHECK_HIP(hipMemcpy(&st, d_state, sizeof(st), hipMemcpyDeviceToHost));
+    EXPECT(st.loss_scale == 64.0f && st.inv_scale == 1.0f / 64.0f && st.unskipped == 1 && st.skipped_steps == 0);
+    /* second clean step: the window is reached, the scale doubles */
+    CHECK_RG(rg_step_begin_scaled(plan, &d_state->inv_scale, NULL));
+    CHECK_RG(rg_step_decide(plan, max_norm, RG_STEP_DEFAULT, NULL));
+    CHECK_RG(rg_scaler_update(d_state, d_result, RG_SCALER_DYNAMIC | RG_SCALER_TRUNCATE, device, NULL));
+    CHECK_HIP(hipDeviceSynchronize());
+    CHECK_HIP(hipMemcpy(&st, d_state, sizeof(st), hipMemcpyDeviceToHost));
+    EXPECT(st.loss_scale == 128.0f && st.inv_scale == 1.0f / 128.0f && st.unskipped == 0);
+    /* an inf: flagged with the new scale in use, the step skipped, the scale halved */
+    {
+      const uint16_t inf_bits = 0xff80; /* -inf */
+      CHECK_HIP(hipMemcpy(d_src + 2 * 5, &inf_bits, 2, hipMemcpyHostToDevice));
+      CHECK_RG(rg_step_begin_scaled(plan, &d_state->inv_scale, NULL));
+      CHECK_RG(rg_step_decide(plan, max_norm, RG_STEP_DEFAULT, NULL));
+      CHECK_RG(rg_scaler_update(d_state, d_result, RG_SCALER_DYNAMIC | RG_SCALER_TRUNCATE, device, NULL));
+      CHECK_RG(rg_read_result(plan, &res, NULL));
+      EXPECT(res.overflow == 1 && res.skipped == 1);
+      CHECK_HIP(hipMemcpy(&st, d_state, sizeof(st), hipMemcpyDeviceToHost));
+      EXPECT(st.loss_scale == 64.0f && st.unskipped == 0 && st.skipped_steps == 1);
+      CHECK_HIP(hipMemcpy(d_src + 2 * 5, &h_src[5], 2, hipMemcpyHostToDevice));
+    }
+    EXPECT(rg_scaler_update(d_state, NULL, RG_SCALER_DYNAMIC, device, NULL) == RG_EINVAL);
+    EXPECT(rg_scaler_update(d_state, d_result, 64, device, NULL) == RG_EINVAL);
+    CHECK_HIP(hipFree(d_state));
+  }
+
   /* ---- segment layout and a cast copy (the ZeRO unflatten), then errors as status codes */
   {
     EXPECT(rg_aligned_numel(1000, 2, 8) == 1024);
