@@ -296,7 +296,7 @@ def run_overflow_host_gate(w: StepWorkload, steps: int, warmup: int) -> dict:
     n, s, d = w.n, w.s, w.d
     moved = s * n if res.overflow else (2 * s + d) * n
     roof = roofline("pass_kernel<reduce, streaming>", s * n, dev_s, measured_traffic("overflow_host_gate", w.key, "pass_kernel<reduce>"),
-                    note="launch time = whole step from device events (read pass + finalize + the host's read of the flag)")
+                    note="launch time = whole step from device events (read pass + reduce + decide + the host's read of the flag)")
     return entry(w.key, "overflow_host_gate", wall, moved, roof, overflow=int(res.overflow), steps=steps,
                  note="bytes = what the step moves: s*N when it is skipped")
 
@@ -588,7 +588,7 @@ def bench_optimizer(args, key, torch, dev) -> dict:
     else:
         bytes_per_elem = (16 + 12 + 2) if adam else (8 + 4 + 2)
     step_bytes = bytes_per_elem * n
-    kernel = ("pass_kernel<reduce> + finalize + optim_kernel<adam>, all launches of a step" if direct
+    kernel = ("pass_kernel<reduce> + reduce + decide + optim_kernel<adam>, all launches of a step" if direct
               else f"optim_kernel<{args.op}, streaming>")
     out = {
         "metric": f"achieved HBM GB/s for the multi-tensor {args.op} step with model copy-back",

@@ -380,7 +380,7 @@ int rg_optim_set_grad_scale_source(rg_optim* opt, const float* grad_scale_dev);
  * TimeCounter around whole calls, src/comp/TimeCounter.cpp:10-27).  With `slots` > 0 every
  * rg_fused_step records HIP events on its stream around its three kernels into the next
  * slot of a ring; slots == 0 switches it off.  rg_plan_read_timing waits for that slot and
- * returns milliseconds: ms[0] reduce pass, ms[1] finalize, ms[2] write pass, ms[3] whole step.
+ * returns milliseconds: ms[0] reduce pass, ms[1] reduce + decide (the partial sums, the decision), ms[2] write pass, ms[3] whole step.
  * slot counts fused steps since timing was enabled, modulo `slots`.
  * A negative `slots` brackets only the write pass (two records per step instead of four, for
  * measurements where the records' own cost matters); ms[0], ms[1], ms[3] then read -1.

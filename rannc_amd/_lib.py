@@ -287,7 +287,7 @@ class Plan:
         check(lib.rg_plan_timing_stride(self._handle, stride))
 
     def read_timing(self, slot: int) -> List[float]:
-        """[reduce pass, finalize, write pass, whole step] in milliseconds."""
+        """[reduce pass, reduce + decide, write pass, whole step] in milliseconds."""
         ms = (C.c_float * 4)()
         check(lib.rg_plan_read_timing(self._handle, slot, ms))
         return list(ms)
