@@ -963,6 +963,10 @@ RG_API int rg_zero(rg_plan* p, void* stream) {
   PassArgs a = pass_args(p, 1.0f);
   a.zero_fill = 1;
   split_for_write(p, a);
+  // A write-only pass wants each XCD to fill runs of consecutive tiles, whatever order the plan's copies prefer
+  // (measured on MI355X: BERT-large's bucket 83 % of peak round robin, 91.5 % with runs of 64 tiles, 90.6 % with
+  // runs of 256, 86 % with contiguous eighths; the ResNet's 83.7 / 87.2 / 87.8 / 82.5 %).
+  a.xcd_run = kZeroXcdRun;
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }

@@ -37,12 +37,19 @@ __global__ __launch_bounds__(256) void ceiling_read_kernel(const char* src, int6
 
 // The writing passes' shape: 128 threads, two steps per block, 16 bytes per lane and step on the
 // wider side (one 4 KiB page of fp32 per block).
-// kind 1: fill (write only)   2: fp32 copy   3: bf16 -> fp32 widening copy   4: four fp32 streams
+// kind 1: fill (write only, XCDs filling runs of 64 tiles)   2: fp32 copy   3: bf16 -> fp32 widening copy   4: four fp32 streams
 // read, three of them written in place (Adam's pattern)   5: fp32 copy with plain `nt` stores
 // 6: kind 4 plus the bf16 model copy as an eighth stream (the optimizer step under mixed precision)
 template <int KIND>
 __global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, char* a2, char* a3, char* a4, int64_t nvec) {
-  const int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  unsigned bid = blockIdx.x;
+  if constexpr (KIND == 1) {
+    // a write-only kernel is fastest when each XCD fills runs of consecutive tiles (rg_zero's order: runs of 64)
+    const unsigned nb = gridDim.x, x = bid & 7u, q = bid >> 3, R = (unsigned)kZeroXcdRun, group = 8u * R;
+    const unsigned g = bid / group;
+    if ((g + 1) * group <= nb) bid = g * group + x * R + (q % R);
+  }
+  const int64_t base = (int64_t)bid * 256 + threadIdx.x;
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int64_t i = base + u * 128;

@@ -233,6 +233,7 @@ __device__ __forceinline__ uint32_t load_u32(const char* p) { return *(const RG_
 __device__ __forceinline__ uint32_t load_u16(const char* p) { return (uint32_t)*(const RG_GLOBAL unsigned short*)p; }
 __device__ __forceinline__ void store_u32(char* p, uint32_t v) { *(RG_GLOBAL uint32_t*)p = v; }
 __device__ __forceinline__ void store_u16(char* p, uint32_t v) { *(RG_GLOBAL unsigned short*)p = (unsigned short)v; }
+__device__ __forceinline__ void store_u8(char* p, uint32_t v) { *(RG_GLOBAL unsigned char*)p = (unsigned char)v; }
 
 template <int DT> __device__ __forceinline__ bool nonfinite_at(const char* p) {
   return (load_u32(p) & 0x7f800000u) == 0x7f800000u;

@@ -100,6 +100,7 @@ constexpr unsigned kReducePassLdsBytes = 32768;   // dynamic LDS of the streamin
 // bf16 gradients into fp32: 79.6 -> 83.8 % of peak, the ResNet's fp32 into fp32: 79.3 -> 81.7 %.  The pass that also
 // sums (rg_unscale_accumulate) holds twelve blocks by its register count already (ten gain on flat same-width data
 // but lose on the ResNet's many small tensors); plain writing passes lose from the first block taken away.
+constexpr int kZeroXcdRun = 64;                      // rg_zero: tiles of a run one XCD fills (see rg_zero)
 constexpr unsigned kAccSameWidthLdsBytes = 16384;   // 10 resident blocks
 constexpr unsigned kAccMixedWidthLdsBytes = 13600;  // 12 resident blocks
 constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan
