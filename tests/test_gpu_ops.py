@@ -354,3 +354,34 @@ def test_plan_tune_changes_only_the_time():
     p2.tune()
     assert torch.equal(t, keep)
     p2.close()
+
+
+@pytest.mark.parametrize("nbytes", [0, 1, 15, 16, 17, 127, 128, 129, 4095, 4096, 4097, 8 * 4096 * 64 + 5, (1 << 20) + 3])
+@pytest.mark.parametrize("offset", [0, 1, 2, 16, 127, 129])
+def test_fill_zero_writes_exactly_its_bytes(nbytes, offset):
+    """``rg_fill_zero`` over a flat byte range at any address: every byte of the range is zero afterwards and no
+    byte outside it is touched (tiles are laid out from the first 128-byte boundary; the bytes before it and
+    behind the last whole 16 are written one at a time)."""
+    from rannc_amd import _lib
+    from rannc_amd.multi_tensor import stream_handle
+    guard = 256
+    arena = torch.full((guard + offset + nbytes + guard,), 0xAB, dtype=torch.uint8, device=DEV)
+    _lib.fill_zero(arena.data_ptr() + guard + offset, nbytes, 0, stream_handle(torch.device(DEV)))
+    torch.cuda.synchronize()
+    lo, hi = guard + offset, guard + offset + nbytes
+    assert int(arena[lo:hi].count_nonzero()) == 0
+    assert int((arena[:lo] == 0xAB).sum()) == lo
+    assert int((arena[hi:] == 0xAB).sum()) == arena.numel() - hi
+
+
+def test_fill_zero_of_a_streaming_size():
+    """Above 256 MiB the fill uses streaming stores; same contract."""
+    from rannc_amd import _lib
+    from rannc_amd.multi_tensor import stream_handle
+    nbytes, offset, guard = (300 << 20) + 5, 3, 256
+    arena = torch.full((guard + offset + nbytes + guard,), 0x5C, dtype=torch.uint8, device=DEV)
+    _lib.fill_zero(arena.data_ptr() + guard + offset, nbytes, 0, stream_handle(torch.device(DEV)))
+    torch.cuda.synchronize()
+    lo, hi = guard + offset, guard + offset + nbytes
+    assert int(arena[lo:hi].count_nonzero()) == 0
+    assert int((arena[:lo] == 0x5C).sum()) == lo and int((arena[hi:] == 0x5C).sum()) == guard
