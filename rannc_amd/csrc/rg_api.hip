@@ -28,6 +28,12 @@ void set_error(const char* fmt, ...) {
 
 using namespace rg;
 
+// Block order of the read-only pass (PassArgs::xcd_run).  Measured on MI355X: round robin loses 6 % on 2.5e9 elements;
+// runs of 16 to 1024 chunks per XCD and one contiguous eighth per XCD are within 1 % of each other, the eighths
+// ahead by 0.5-1 % on all three workloads tried.
+#ifndef RG_XCD_REDUCE_RUN
+#define RG_XCD_REDUCE_RUN (-1)
+#endif
 struct rg_plan {
   int device = 0;
   int n_tensors = 0;
@@ -38,7 +44,7 @@ struct rg_plan {
   bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
   int64_t write_tile_elems = kWriteTileElems;
   unsigned accumulate_lds = 0;   // unused dynamic LDS of rg_accumulate's pass (resident-block cap)
-  int xcd_reduce = 64;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
+  int xcd_reduce = RG_XCD_REDUCE_RUN;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
   int xcd_write = 0;                 //   ... when every source sits on the line grid of its destination
   int xcd_write_offgrid = 256;       //   ... when some source does not (see fill_chunk_records)
   float begun_inv_scale = 0.0f;  // inv_scale of the last rg_step_begin, 0 = none pending
@@ -925,7 +931,7 @@ RG_API int rg_fused_step_static(const void* src_dev, void* dst_dev, int64_t nume
   a.tile_elems = (int32_t)chunk;
   a.tiles_per_chunk = 1;
   a.scale = inv_scale;
-  a.xcd_run = 64;
+  a.xcd_run = RG_XCD_REDUCE_RUN;
   RG_HIP(launch_pass(kModeReduce, a, streaming, s));
 
   ReduceArgs f;
