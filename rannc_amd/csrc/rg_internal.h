@@ -115,7 +115,7 @@ struct alignas(16) Partial {
   int32_t bad;
   int32_t pad;
 };
-constexpr int kWaveSlotsPerTile = kWriteThreads / 64;   // partials one tile of a pass that sums while it writes leaves
+constexpr int kWaveSlotsPerTile = 1;   // partials one tile of a pass that sums while it writes leaves (its wavefronts meet in LDS)
 
 // From partials to the decision in two launches.  The partials of a tensor are cut into segments of whole chunks
 // (kSegmentChunks each; more for a tensor that would otherwise have over kMaxSegmentsPerTensor of them): one block
@@ -136,7 +136,7 @@ struct PassArgs {
   int64_t single_head;           // elements before the first aligned chunk boundary
   int32_t xcd_run;               // block -> XCD mapping, see pass_kernel
   int32_t peel_heads;            // writing passes: some destination starts off a boundary
-  Partial* partials;             // read-only pass: [n_chunks]; pass that sums while it writes: one per wavefront of every tile
+  Partial* partials;             // read-only pass: [n_chunks]; pass that sums while it writes: one per tile
   const StepResult* result;      // non-null: take coef / overflow gate from the device
   int64_t n_chunks;
   int32_t tile_elems;            // elements one block handles (== chunk_elems unless the pass splits chunks)
@@ -164,7 +164,7 @@ struct ReduceArgs {
   rg_step_result* result_copy;        // optional second place the decision is written to (caller's memory)
   int32_t n_tensors;
   int32_t n_segments;
-  int32_t partials_per_chunk;         // 1 after the read-only pass, else tiles per chunk * kWaveSlotsPerTile
+  int32_t partials_per_chunk;         // 1 after the read-only pass, else tiles per chunk (* kWaveSlotsPerTile)
   float max_norm;
   int32_t ignore_overflow;            // overflow is reported but neither gates the clip nor the write
 };

@@ -261,8 +261,10 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
   const int start = tile == 0 ? 0 : chunk_head + tile * a.tile_elems;
   int end = tile == a.tiles_per_chunk - 1 ? rec.len : chunk_head + (tile + 1) * a.tile_elems;
   if (end > rec.len) end = rec.len;
-  // A pass that reduces and writes leaves one partial per wavefront (no block-wide combine at
-  // the end of a tile that only lives a few microseconds); a read-only pass one per block.
+  // A pass that reduces and writes leaves one partial per tile, a read-only pass one per chunk.  (Per-wavefront
+  // partials, without the barrier, were the faster form only while every wavefront also sat out a full drain of its
+  // memory counter after its last store; since that wait is gone, one record per tile is 0.5 points faster and
+  // halves what the reduction has to read.)
   constexpr bool kWavePartials = (MODE & kModeReduce) != 0 && (MODE & kModeWrite) != 0;
   constexpr int kSlots = kWavePartials ? kWaveSlotsPerTile : 1;
   if (start >= end) {
@@ -329,8 +331,9 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
     // one by one (the sum can also overflow from finite inputs).
     constexpr int kWaves = T / 64;
     if constexpr (kWavePartials) {
-      // One partial per wavefront: sum and flag leave in one 16-byte store.  A wavefront whose sum is not finite
-      // looks at every element of the tile again (its own elements are strided through it), 64 at a time.
+      // Each wavefront reduces its own lanes; a wavefront whose sum is not finite looks at every element of the
+      // tile again (its own elements are strided through it), 64 at a time.  Sum and flag of the tile leave in
+      // one 16-byte store.
       auto rescan = [&]() -> int {
         int mine = 0;
         if (sp != nullptr) {
@@ -344,12 +347,28 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
         }
         return __any(mine) ? 1 : 0;
       };
-      Partial* const slot = &a.partials[slot_id * kSlots + (threadIdx.x >> 6)];
       double s = (((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3])) +
                  (((double)acc[4] + (double)acc[5]) + ((double)acc[6] + (double)acc[7]));
       s = wave_total(s);
       const int bad = !(fabs(s) <= 1.79769313486231570e308) ? rescan() : 0;
-      if ((threadIdx.x & 63) == 0) *slot = Partial{s, bad, 0};
+      // the wavefronts of the tile meet in LDS: one record per tile, added in wavefront order
+      __shared__ double wave_sum[kWaves];
+      __shared__ int wave_bad[kWaves];
+      if ((threadIdx.x & 63) == 0) {
+        wave_sum[threadIdx.x >> 6] = s;
+        wave_bad[threadIdx.x >> 6] = bad;
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        double total = wave_sum[0];
+        int any = wave_bad[0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) {
+          total += wave_sum[w];
+          any |= wave_bad[w];
+        }
+        a.partials[slot_id] = Partial{total, any, 0};
+      }
     } else {
       // One partial per block: the 8 sums of the thread, the 64 lanes of the wavefront by DPP row scans, the
       // wavefronts through LDS in index order.  Everything past the per-thread fp32 sums is double.
