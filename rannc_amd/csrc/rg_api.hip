@@ -291,7 +291,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   const size_t nt = (size_t)(n > 0 ? n : 1), nc = (size_t)(p->n_chunks > 0 ? p->n_chunks : 1);
   const size_t ns = (size_t)(p->n_segments > 0 ? p->n_segments : 1);
   const size_t o_chunks = carve(nc * sizeof(ChunkRec));
-  // a pass that sums while it writes leaves one partial per wavefront of every tile
+  // a pass that sums while it writes leaves one partial per tile
   if (p->write_tile_elems < kMinWriteTileElems) p->write_tile_elems = kMinWriteTileElems;
   const size_t max_tiles = (size_t)((p->chunk_elems + p->write_tile_elems - 1) / p->write_tile_elems);
   const size_t o_partials = carve(nc * max_tiles * (size_t)kWaveSlotsPerTile * sizeof(Partial));
@@ -468,9 +468,8 @@ static hipError_t launch_scale_if_clipped(const rg_plan* p, hipStream_t s) {
   return launch_gated_pass(b, p->streaming, s);
 }
 
-// One pass that both reduces and writes, over tiles of each chunk: every wavefront of every
-// tile leaves its own partial sum; two small launches (one for small plans) turn them into the
-// per-tensor norms and the decision.
+// One pass that both reduces and writes, over tiles of each chunk: every tile leaves its own partial sum; two
+// small launches (one for small plans) turn them into the per-tensor norms and the decision.
 static int tiled_reduce_write(rg_plan* p, PassArgs& a, int mode, hipStream_t s, float max_norm = 0.0f,
                               int ignore_overflow = 0, hipEvent_t after_pass = nullptr) {
   split_for_write(p, a);
