@@ -28,7 +28,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 HEADLINE = "c3_bert_enlarged"
 
 FUSED_OPS = ("fused_step", "fused_step_noclip", "fused_step_noclip_2pass", "overflow_host_gate", "unscale_pack",
-             "copy_back", "unflatten_back", "grad_norm", "zero", "accumulate", "unscale_accumulate", "clip_in_place",
+             "copy_back", "unflatten_back", "grad_norm", "zero", "zero_bucket", "accumulate", "unscale_accumulate", "clip_in_place",
              "consolidate", "zero_staging_pack")
 C5_OPS = ("c5_unflatten", "c5_master_cast", "c5_copy_back", "c5_repack")
 OPTIM_OPS = ("adam", "sgd", "adam_from_model_grads")
@@ -313,6 +313,10 @@ def run_plan_op(w: StepWorkload, op: str, steps: int, warmup: int) -> dict:
         fn, nbytes, kernel = w.plan.grad_norm, s * n, "pass_kernel<reduce>"
     elif op == "zero":
         fn, nbytes, kernel = w.plan.zero, d * n, "pass_kernel<write> (zero fill)"
+    elif op == "zero_bucket":
+        # clearParamGrads on consolidated gradients: the bucket itself is cleared, as one flat range (rg_fill_zero)
+        from rannc_amd.multi_tensor import fill_zero_
+        fn, nbytes, kernel = (lambda: fill_zero_(w.bucket)), d * n, "fill_zero_kernel"
     elif op in ("accumulate", "unscale_accumulate"):
         # dst += src * scale: the destination is read and written; the second form also reports flag and norm
         w.bucket.zero_()
@@ -944,12 +948,12 @@ def main() -> int:
             ("c3_bert_enlarged", "fused_step_noclip", args.steps), ("c3_bert_enlarged", "unscale_pack", args.steps),
             ("c2_bert_large", "fused_step", sub), ("c2_bert_large", "fused_step_noclip", sub),
             ("c2_bert_large", "fused_step_noclip_2pass", sub), ("c2_bert_large", "unscale_pack", sub),
-            ("c2_bert_large", "copy_back", sub), ("c2_bert_large", "zero", sub), ("c2_bert_large", "grad_norm", sub),
+            ("c2_bert_large", "copy_back", sub), ("c2_bert_large", "zero", sub), ("c2_bert_large", "zero_bucket", sub), ("c2_bert_large", "grad_norm", sub),
             ("c2_bert_large", "accumulate", sub), ("c2_bert_large", "unscale_accumulate", sub),
             ("c2_bert_large", "clip_in_place", sub), ("c2_bert_large", "consolidate", sub),
             ("c2_bert_large", "zero_staging_pack", sub),
             ("c4_resnet152x2", "fused_step", sub), ("c4_resnet152x2", "fused_step_noclip", sub),
-            ("c4_resnet152x2", "unscale_pack", sub), ("c4_resnet152x2", "zero", sub), ("c4_resnet152x2", "grad_norm", sub),
+            ("c4_resnet152x2", "unscale_pack", sub), ("c4_resnet152x2", "zero", sub), ("c4_resnet152x2", "zero_bucket", sub), ("c4_resnet152x2", "grad_norm", sub),
             ("c4_resnet152x2", "accumulate", sub), ("c4_resnet152x2", "unscale_accumulate", sub),
             ("c4_resnet152x2", "clip_in_place", sub), ("c4_resnet152x2", "consolidate", sub),
             ("c4_resnet152x2", "zero_staging_pack", sub),
