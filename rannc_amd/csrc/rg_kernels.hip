@@ -20,6 +20,7 @@
 //
 // The work is purely bandwidth bound (a few ALU ops per element): no LDS staging and no
 // MFMA.  LDS is used only for the 4-wavefront combine of the partial sums.
+#include <atomic>
 #include <cstdlib>
 #include <type_traits>
 
@@ -604,15 +605,28 @@ __global__ __launch_bounds__(kDecideThreads) void reduce_small_kernel(ReduceArgs
 // (two 16-byte stores per lane), each XCD filling runs of kZeroXcdRun consecutive tiles; the bytes before that
 // boundary and behind the last whole 16 are written one at a time by block 0.  (A grid-stride loop over the same
 // bytes ran at 63-65 % of peak where this runs at 90 % and more.)
+//
+// Pacing.  A wavefront of this kernel has nothing to wait for - it issues its two stores and ends - so the compute
+// units hand stores to the memory system as fast as wavefronts can be launched, faster than HBM retires them, and
+// the fill then runs at 85-88 % of peak.  Holding every wavefront for `delay_ticks` of the constant-rate wall clock
+// before its stores makes the 32 wavefront slots of a compute unit a rate limiter (64 KiB per wavefront lifetime);
+// measured on MI355X over 1-4 GiB, by delay: none 85-88 %, 1.25 us 89 %, 1.4-1.5 us 95-97 %, 1.55 us 94 %, 1.7 us
+// 88 %, and falling in proportion from there (the limiter then sits below what HBM takes).  The wall clock, not
+// s_sleep's shader cycles, measures the delay so that the rate does not move with the shader clock.  Passes that
+// load before they store are paced by their loads and only lose from such a delay.
 constexpr int kFillTileVecs = 4096 / 16;
 template <bool NT>
-__global__ __launch_bounds__(kWriteThreads) void fill_zero_kernel(char* p, int64_t nbytes, int64_t head) {
+__global__ __launch_bounds__(kWriteThreads) void fill_zero_kernel(char* p, int64_t nbytes, int64_t head, int delay_ticks) {
   unsigned bid = blockIdx.x;
   {
     const unsigned nb = gridDim.x, x = bid & 7u, q = bid >> 3;
     const unsigned R = (unsigned)kZeroXcdRun, group = 8u * R;
     const unsigned g = bid / group;
     if ((g + 1) * group <= nb) bid = g * group + x * R + (q % R);   // the ragged last group keeps its order
+  }
+  if (delay_ticks > 0) {
+    const uint64_t t_end = wall_clock64() + (uint64_t)delay_ticks;
+    while (wall_clock64() < t_end) __builtin_amdgcn_s_sleep(1);
   }
   const int64_t nvec = (nbytes - head) / 16;
   const int64_t tail0 = head + nvec * 16;
@@ -697,6 +711,31 @@ hipError_t launch_decide(const ReduceArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// kFillDelayNs in ticks of the current device's wall clock (0 when its rate cannot be read: the fill then runs unpaced).
+#ifndef RG_FILL_DELAY_NS
+#define RG_FILL_DELAY_NS 1450
+#endif
+constexpr int kFillDelayNs = RG_FILL_DELAY_NS;
+constexpr int kMaxDevices = 64;
+static int fill_delay_ticks() {
+  static std::atomic<int> cached[kMaxDevices];   // 0: not asked yet; -1: unknown rate
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int t = cached[dev].load(std::memory_order_relaxed);
+  if (t == 0) {
+    int khz = 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0) {
+      (void)hipGetLastError();
+      t = -1;
+    } else {
+      t = (int)(((int64_t)khz * kFillDelayNs + 500000) / 1000000);
+      if (t < 1) t = -1;
+    }
+    cached[dev].store(t, std::memory_order_relaxed);
+  }
+  return t > 0 ? t : 0;
+}
+
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream) {
   if (nbytes <= 0) return hipSuccess;
   char* p = reinterpret_cast<char*>(dst);
@@ -706,8 +745,12 @@ hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream) {
   int64_t blocks = (nvec + kFillTileVecs - 1) / kFillTileVecs;
   if (blocks < 1) blocks = 1;   // block 0 writes the bytes outside the vectors
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  if (nbytes > ((int64_t)256 << 20)) hipLaunchKernelGGL(fill_zero_kernel<true>, dim3((unsigned)blocks), dim3(kWriteThreads), 0, stream, p, nbytes, head);
-  else hipLaunchKernelGGL(fill_zero_kernel<false>, dim3((unsigned)blocks), dim3(kWriteThreads), 0, stream, p, nbytes, head);
+  // Paced only where the stores go through to HBM: up to the 256 MiB of the memory-side cache the unpaced fill
+  // is the faster one (192 MiB: 98 % of HBM's peak rate unpaced, 90 % paced), and a small fill would just start late.
+  const bool streaming = nbytes > ((int64_t)256 << 20);
+  const int delay = streaming ? fill_delay_ticks() : 0;
+  if (streaming) hipLaunchKernelGGL(fill_zero_kernel<true>, dim3((unsigned)blocks), dim3(kWriteThreads), 0, stream, p, nbytes, head, delay);
+  else hipLaunchKernelGGL(fill_zero_kernel<false>, dim3((unsigned)blocks), dim3(kWriteThreads), 0, stream, p, nbytes, head, delay);
   return hipGetLastError();
 }
 
