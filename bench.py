@@ -423,7 +423,7 @@ def run_ceilings(steps: int, warmup: int, nbytes: int = 1 << 30) -> list:
     arrays = [torch.empty(nbytes // 4, dtype=torch.float32, device=dev).fill_(1.0) for _ in range(5)]
     ptrs = [a.data_ptr() for a in arrays]
     out = []
-    for name, kind, moved in (("read", 0, 1.0), ("fill", 1, 1.0), ("copy_f32", 2, 2.0), ("copy_f32_nt", 5, 2.0),
+    for name, kind, moved in (("read", 0, 1.0), ("fill", 1, 1.0), ("fill_paced", 8, 1.0), ("copy_f32", 2, 2.0), ("copy_f32_nt", 5, 2.0),
                               ("widen_bf16_f32", 3, 1.5), ("adam_streams", 4, 7.0), ("adam_streams_bf16_copy", 6, 7.5),
                               ("adam_streams_bf16_copy_step_shape", 7, 7.5)):
         def fn():

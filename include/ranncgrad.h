@@ -402,7 +402,8 @@ int rg_plan_read_timing(rg_plan* plan, int slot, float ms[4]);
  *   kind 4  Adam's streams        arrays: p, g, m, v [nbytes each]; p, m, v rewritten in place
  *   kind 5  kind 2 with the compiler's plain nontemporal stores instead of the write passes' cache policy
  *   kind 6  kind 4 + a bf16 copy  arrays: p, g, m, v [nbytes each], copy[nbytes / 2] written (the step under mixed precision)
- *   kind 7  kind 6 in the optimizer step's launch shape (256 threads over 4096 elements, four vectors per array in flight) */
+ *   kind 7  kind 6 in the optimizer step's launch shape (256 threads over 4096 elements, four vectors per array in flight)
+ *   kind 8  kind 1 paced as rg_fill_zero paces a fill above 256 MiB (every wavefront waits 1.45 us before it stores) */
 int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, int64_t nbytes, int device, void* stream);
 
 #ifdef __cplusplus

@@ -40,14 +40,19 @@ __global__ __launch_bounds__(256) void ceiling_read_kernel(const char* src, int6
 // kind 1: fill (write only, XCDs filling runs of 64 tiles)   2: fp32 copy   3: bf16 -> fp32 widening copy   4: four fp32 streams
 // read, three of them written in place (Adam's pattern)   5: fp32 copy with plain `nt` stores
 // 6: kind 4 plus the bf16 model copy as an eighth stream (the optimizer step under mixed precision)
+// 8: kind 1 with every wavefront held for `delay_ticks` of the wall clock before its stores (rg_fill_zero's pacing)
 template <int KIND>
-__global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, char* a2, char* a3, char* a4, int64_t nvec) {
+__global__ __launch_bounds__(128) void ceiling_write_kernel(char* a0, char* a1, char* a2, char* a3, char* a4, int64_t nvec, int delay_ticks) {
   unsigned bid = blockIdx.x;
   if constexpr (KIND == 1) {
     // a write-only kernel is fastest when each XCD fills runs of consecutive tiles (rg_zero's order: runs of 64)
     const unsigned nb = gridDim.x, x = bid & 7u, q = bid >> 3, R = (unsigned)kZeroXcdRun, group = 8u * R;
     const unsigned g = bid / group;
     if ((g + 1) * group <= nb) bid = g * group + x * R + (q % R);
+    if (delay_ticks > 0) {   // kind 8: the flat fill's pacing
+      const uint64_t t_end = wall_clock64() + (uint64_t)delay_ticks;
+      while (wall_clock64() < t_end) __builtin_amdgcn_s_sleep(1);
+    }
   }
   const int64_t base = (int64_t)bid * 256 + threadIdx.x;
 #pragma unroll
@@ -125,8 +130,8 @@ __global__ __launch_bounds__(256) void ceiling_adam_shape_kernel(char* a0, char*
 using namespace rg;
 
 RG_API int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, int64_t nbytes, int device, void* stream) {
-  static const int need[8] = {2, 1, 2, 2, 4, 2, 5, 5};
-  if (kind < 0 || kind > 7 || arrays_dev == nullptr || n_arrays < need[kind] || nbytes < 16 || nbytes % 16 != 0) {
+  static const int need[9] = {2, 1, 2, 2, 4, 2, 5, 5, 1};
+  if (kind < 0 || kind > 8 || arrays_dev == nullptr || n_arrays < need[kind] || nbytes < 16 || nbytes % 16 != 0) {
     set_error("rg_ceiling_kernel: bad arguments (kind %d, %d arrays, %lld bytes)", kind, n_arrays, (long long)nbytes);
     return RG_EINVAL;
   }
@@ -169,12 +174,13 @@ RG_API int rg_ceiling_kernel(int kind, void* const* arrays_dev, int n_arrays, in
   }
   const dim3 grid((unsigned)blocks), block(128);
   switch (kind) {
-    case 1: hipLaunchKernelGGL(ceiling_write_kernel<1>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
-    case 2: hipLaunchKernelGGL(ceiling_write_kernel<2>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
-    case 3: hipLaunchKernelGGL(ceiling_write_kernel<3>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
-    case 4: hipLaunchKernelGGL(ceiling_write_kernel<4>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
-    case 6: hipLaunchKernelGGL(ceiling_write_kernel<6>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
-    default: hipLaunchKernelGGL(ceiling_write_kernel<5>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec); break;
+    case 1: hipLaunchKernelGGL(ceiling_write_kernel<1>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec, 0); break;
+    case 8: hipLaunchKernelGGL(ceiling_write_kernel<1>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec, fill_delay_ticks()); break;
+    case 2: hipLaunchKernelGGL(ceiling_write_kernel<2>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec, 0); break;
+    case 3: hipLaunchKernelGGL(ceiling_write_kernel<3>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec, 0); break;
+    case 4: hipLaunchKernelGGL(ceiling_write_kernel<4>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec, 0); break;
+    case 6: hipLaunchKernelGGL(ceiling_write_kernel<6>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec, 0); break;
+    default: hipLaunchKernelGGL(ceiling_write_kernel<5>, grid, block, 0, s, a[0], a[1], a[2], a[3], a[4], nvec, 0); break;
   }
   RG_HIP(hipGetLastError());
   return RG_OK;

@@ -178,6 +178,8 @@ hipError_t launch_reduce(const ReduceArgs& a, int64_t n_chunks, hipStream_t stre
 // segment sums (left by an earlier launch_reduce) -> per-tensor norms -> decision for a.max_norm
 hipError_t launch_decide(const ReduceArgs& a, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
+// Ticks of the current device's wall clock that a wavefront of a large flat fill waits before it stores (0: unknown rate).
+int fill_delay_ticks();
 
 void set_error(const char* fmt, ...);
 

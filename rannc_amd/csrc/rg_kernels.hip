@@ -717,7 +717,7 @@ hipError_t launch_decide(const ReduceArgs& a, hipStream_t stream) {
 #endif
 constexpr int kFillDelayNs = RG_FILL_DELAY_NS;
 constexpr int kMaxDevices = 64;
-static int fill_delay_ticks() {
+int fill_delay_ticks() {
   static std::atomic<int> cached[kMaxDevices];   // 0: not asked yet; -1: unknown rate
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
