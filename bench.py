@@ -312,7 +312,17 @@ def run_plan_op(w: StepWorkload, op: str, steps: int, warmup: int) -> dict:
     elif op == "grad_norm":
         fn, nbytes, kernel = w.plan.grad_norm, s * n, "pass_kernel<reduce>"
     elif op == "zero":
-        fn, nbytes, kernel = w.plan.zero, d * n, "pass_kernel<write> (zero fill)"
+        # clearParamGrads without consolidation: one separately allocated tensor per gradient, each cleared where it lies
+        # (rg_zero takes the table-driven pass unless the tensors happen to lie back to back: those it clears as one range)
+        outs = [torch.empty_like(g) for g in w.grads]     # stand-ins: the workload's gradients feed the other operations
+        plan = TensorPlan([None] * len(outs), outs)
+        cleanup.append(plan)
+        end, flat = None, True
+        for g in outs:
+            if g.numel():
+                flat = flat and end in (None, g.data_ptr())
+                end = g.data_ptr() + g.numel() * g.element_size()
+        fn, nbytes, kernel = plan.zero, s * n, "fill_zero_kernel" if flat else "pass_kernel<write> (zero fill)"
     elif op == "zero_bucket":
         # clearParamGrads on consolidated gradients: the bucket itself is cleared, as one flat range (rg_fill_zero)
         from rannc_amd.multi_tensor import fill_zero_

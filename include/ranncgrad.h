@@ -219,7 +219,9 @@ int rg_scale_cast(rg_plan* plan, float scale, void* stream);
 int rg_scale_cast_single(const void* src_dev, void* dst_dev, int64_t numel, int src_dtype, int dst_dtype,
                          float scale, int device, void* stream);
 
-/* dst = 0 for every tensor.  ParamStorage::clearParamGrads, src/comp/ParamStorage.cpp:540-557. */
+/* dst = 0 for every tensor.  ParamStorage::clearParamGrads, src/comp/ParamStorage.cpp:540-557.
+ * Destinations that follow each other back to back in plan order (the views of a bucket) are cleared as one flat range,
+ * as rg_fill_zero would; scattered ones through the plan's table. */
 int rg_zero(rg_plan* plan, void* stream);
 
 /* Fill `nbytes` bytes at dst_dev with zero (bucket / staging clears:

@@ -65,6 +65,48 @@ def test_same_dtype_copy_preserves_every_bit_pattern():
     assert torch.equal(dst.cpu().view(torch.int32), f)
 
 
+def test_zero_over_back_to_back_destinations_and_after_they_move_apart():
+    """Destinations that lie back to back in plan order (the views of a bucket, of mixed widths here) are cleared as one
+    flat range; once an update moves one of them away the table-driven pass takes over.  Either way exactly the
+    destinations' bytes change."""
+    arena = torch.full((1 << 20,), 0x55, dtype=torch.uint8, device=DEV)
+    specs = [(torch.float16, 1002), (torch.float32, 0), (torch.float32, 30000), (torch.bfloat16, 6), (torch.float32, 4099)]
+
+    def views(start, gap_before=None, gap=0):
+        out, o = [], start
+        for i, (dt, n) in enumerate(specs):
+            if i == gap_before:
+                o += gap
+            es = torch.empty((), dtype=dt).element_size()
+            out.append(arena[o:o + n * es].view(dt))
+            o += n * es
+        return out, o
+
+    def check(dsts):
+        torch.cuda.synchronize()
+        covered = torch.zeros(arena.numel(), dtype=torch.bool)
+        base = arena.data_ptr()
+        for d in dsts:
+            covered[d.data_ptr() - base:d.data_ptr() - base + d.numel() * d.element_size()] = True
+        got = arena.cpu()
+        assert bool((got[covered] == 0).all()) and bool((got[~covered] == 0x55).all())
+        arena.fill_(0x55)
+
+    dsts, _ = views(4)                                    # 4-byte aligned start, off the 128-byte grid
+    plan = TensorPlan([None] * len(dsts), dsts, chunk_elems=2048)
+    plan.zero()
+    check(dsts)
+    moved, _ = views(4, gap_before=3, gap=64)            # the last two move 64 bytes up: no longer one range
+    plan.update(dsts=moved)
+    plan.zero()
+    check(moved)
+    back, _ = views(260)                                  # one range again, elsewhere
+    plan.update(dsts=back)
+    plan.zero()
+    check(back)
+    plan.close()
+
+
 @pytest.mark.parametrize("dst_name", ["f32", "f16", "bf16"])
 def test_zero_fills_only_the_destinations(dst_name):
     ddt = TORCH_DTYPE[dst_name]
