@@ -320,6 +320,7 @@ RG_API int rg_plan_create(rg_plan** out, int device, int n, const void* const* s
   p->dev_bytes = off;
 
   DeviceGuard guard(device);
+  (void)fill_delay_ticks();   // ask the device for its wall-clock rate here, not on the first large rg_zero (which a caller may be capturing)
   hipError_t e = hipMalloc(reinterpret_cast<void**>(&p->dev_base), p->dev_bytes);
   if (e != hipSuccess) {
     delete p;

@@ -359,3 +359,31 @@ def test_dynamic_loss_scale_on_the_device_replays_from_a_graph():
     assert scales_seen == [50.0, 25.0, 25.0, 12.0, 12.0, 24.0, 24.0]      # written by hand from the schedule
     assert steps_done == 6 and device_scaler().skipped_steps == 2
     plan.close()
+
+
+def test_paced_flat_fill_replays_from_a_graph():
+    """A fill above 256 MiB holds every wavefront for a fixed wall-clock time before its stores (pacing); the kernel
+    reads only the clock, so it can be captured like the others.  Guard bytes around the range stay as they were."""
+    from rannc_amd.multi_tensor import fill_zero_
+    n = (300 << 20) + 24                                   # bytes; the range starts 8 bytes into the allocation
+    arena = torch.full((n + 16,), 0x5A, dtype=torch.uint8, device=DEV)
+    target = arena[8:8 + n]
+    fill_zero_(target)                                     # eager once: also the warm-up
+    torch.cuda.synchronize()
+    assert int(target.max()) == 0 and int(arena[:8].min()) == 0x5A and int(arena[8 + n:].min()) == 0x5A
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fill_zero_(target)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fill_zero_(target)
+    for replay in range(3):
+        arena.fill_(0x5A + replay)                         # eager work between replays; the range must be cleared again
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(target.max()) == 0, f"replay {replay}"
+        assert int(arena[:8].min()) == 0x5A + replay and int(arena[8 + n:].min()) == 0x5A + replay
