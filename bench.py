@@ -182,7 +182,6 @@ class StepWorkload:
         # as a caller does once per plan: the library times its block -> XCD orders on this plan's own tensors
         # (destinations hold zeros here; a real caller tunes before the first step, when they are dead too)
         self.write_order = self.plan.tune()
-        self.read_residency = self.plan.read_residency()
 
     def close(self):
         self.plan.close()
@@ -193,7 +192,7 @@ class StepWorkload:
         return {"workload": self.key, "description": self.cfg.description, "tensors": len(self.grads), "elements": self.n,
                 "src_bytes_per_elem": self.s, "dst_bytes_per_elem": self.d,
                 "chunk_elems": self.plan.plan.chunk_elems, "chunks": self.plan.plan.num_chunks,
-                "tuned_write_order": self.write_order, "tuned_read_residency": self.read_residency}
+                "tuned_write_order": self.write_order}
 
 
 def run_fused_step(w: StepWorkload, steps: int, warmup: int, op: str = "fused_step") -> dict:
@@ -894,7 +893,6 @@ def run_one(args, key: str, op: str, steps: int, warmup: int) -> tuple:
         e = run_plan_op(w, op, steps, warmup)
     if op not in ("copy_back", "unflatten_back", "consolidate", "zero_staging_pack"):
         e.setdefault("tuned_write_order", w.write_order)
-        e.setdefault("tuned_read_residency", w.read_residency)
     desc = w.describe()
     dtype = f"{w.cfg.grad_dtype}->{w.cfg.bucket_dtype} (fp32 arithmetic)"
     w.close()
@@ -988,7 +986,6 @@ def main() -> int:
                 configs.append(run_plan_op(w, op2, st, args.warmup))
             if op2 not in ("copy_back", "unflatten_back", "consolidate", "zero_staging_pack"):      # those run on plans of their own, not tuned
                 configs[-1].setdefault("tuned_write_order", w.write_order)
-                configs[-1].setdefault("tuned_read_residency", w.read_residency)
         if w is not None:
             w.close()
         free, _ = torch.cuda.mem_get_info()

@@ -119,28 +119,20 @@ int64_t rg_plan_total_numel(const rg_plan* plan);
  * plan then hits in cache), -1 = decide from the plan's size (the default). */
 int rg_plan_set_streaming(rg_plan* plan, int mode);
 
-/* Optional: let the library measure, on the plan's own tensors and on `stream`, two things that change the time of
- * its passes and never their results, and keep the faster setting for every later pass of this plan (a setting in
- * use is only given up for one that is more than 1 % faster; candidates are timed in three interleaved rounds; the
- * call waits for the stream):
- *  - for plans large enough to stream: whether the read-only pass (rg_grad_norm, rg_step_begin, pass 1 of
- *    rg_fused_step) runs with five or with all eight 256-thread blocks resident per compute unit - which is faster
- *    differs from one MI355X to the next, not from plan to plan.  This pass writes only the plan's own partial sums;
- *  - for plans whose tensors all have destinations other than their sources: the order in which the writing passes
- *    hand their tiles to the GPU's eight XCDs.  For this the pass `dst = round_dst(float(src))` (what
- *    rg_scale_cast(plan, 1.0) writes) is run under each order the library knows: the destinations are overwritten,
- *    so call it where their contents do not matter yet (right after creating the plan).
- * No counterpart in the reference (it has no kernels to tune).
+/* Optional: choose the order in which the plan's writing passes hand their tiles to the GPU's eight XCDs by
+ * measuring it.  Runs the pass `dst = round_dst(float(src))` (what rg_scale_cast(plan, 1.0) writes) a few times
+ * under each order the library knows (three interleaved rounds), on the plan's own tensors and on `stream`, waits
+ * for them, and keeps the fastest for every later writing pass of this plan - the order in use is only given up
+ * for one that is more than 1 % faster.  The destinations are overwritten, so call it where their
+ * contents do not matter yet (right after creating the plan); in-place plans are left alone.  Results never
+ * depend on the order - only the time does.  No counterpart in the reference (it has no kernels to tune).
  * rg_plan_write_order returns the order in use (0 = round robin, n > 0 = runs of n tiles per XCD, -1 = one
- * contiguous eighth per XCD), rg_plan_read_residency the resident blocks of the read-only pass (5 or 8). */
+ * contiguous eighth per XCD). */
 int rg_plan_tune(rg_plan* plan, void* stream);
 int rg_plan_write_order(const rg_plan* plan);
-int rg_plan_read_residency(const rg_plan* plan);
-/* Set them directly (same encodings; RG_EINVAL outside [-1, 65536], or for blocks other than 5 and 8): for a caller
- * that has measured them on an earlier plan of the same layout and must not have this plan's destinations
- * overwritten by another measurement. */
+/* Set that order directly (same encoding; RG_EINVAL outside [-1, 65536]): for a caller that has measured it on an
+ * earlier plan of the same layout and must not have this plan's destinations overwritten by another measurement. */
 int rg_plan_set_write_order(rg_plan* plan, int order);
-int rg_plan_set_read_residency(rg_plan* plan, int blocks);
 
 /* ---------------------------------------------------------------- per-step operations */
 

@@ -56,8 +56,6 @@ SIGNATURES = {
     "rg_plan_total_numel": (_i64, [_vp]),
     "rg_plan_set_streaming": (_i, [_vp, _i]),
     "rg_plan_tune": (_i, [_vp, _vp]),
-    "rg_plan_read_residency": (_i, [_vp]),
-    "rg_plan_set_read_residency": (_i, [_vp, _i]),
     "rg_plan_write_order": (_i, [_vp]),
     "rg_plan_set_write_order": (_i, [_vp, _i]),
     "rg_fused_step": (_i, [_vp, _f, _f, _i, _vp]),
@@ -211,18 +209,9 @@ class Plan:
         """1 = nontemporal accesses, 0 = plain, -1 = decide from the plan's size."""
         check(lib.rg_plan_set_streaming(self._handle, mode))
 
-    @property
-    def read_residency(self) -> int:
-        """Blocks of the read-only pass resident per compute unit when the plan streams (5 or 8)."""
-        return int(lib.rg_plan_read_residency(self._handle))
-
-    def set_read_residency(self, blocks: int) -> None:
-        check(lib.rg_plan_set_read_residency(self._handle, blocks))
-
     def tune(self, stream: int = 0) -> int:
-        """Measure, on the plan's own tensors, the resident blocks of the read-only pass and the block -> XCD orders
-        of the writing passes, and keep the fastest (the latter overwrites the destinations; waits for the stream).
-        Returns the write order chosen."""
+        """Measure the block -> XCD orders on the plan's own tensors and keep the fastest (overwrites the
+        destinations, waits for the stream).  Returns the order chosen."""
         check(lib.rg_plan_tune(self._handle, _vp(stream)))
         return int(lib.rg_plan_write_order(self._handle))
 

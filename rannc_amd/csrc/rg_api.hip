@@ -44,7 +44,6 @@ struct rg_plan {
   bool streaming = false;   // nontemporal accesses: the data is far larger than the caches
   int64_t write_tile_elems = kWriteTileElems;
   unsigned accumulate_lds = 0;   // unused dynamic LDS of rg_accumulate's pass (resident-block cap)
-  unsigned reduce_lds = 0;       // ... of the read-only pass (0: the default cap; set by rg_plan_tune)
   int xcd_reduce = RG_XCD_REDUCE_RUN;               // block -> XCD mapping of read-only / writing passes (PassArgs::xcd_run)
   int xcd_write = 0;                 //   ... when every source sits on the line grid of its destination
   int xcd_write_offgrid = 256;       //   ... when some source does not (see fill_chunk_records)
@@ -438,7 +437,6 @@ static PassArgs pass_args(const rg_plan* p, float scale) {
   a.tile_elems = (int32_t)p->chunk_elems;
   a.tiles_per_chunk = 1;
   a.peel_heads = p->dst_heads ? 1 : 0;
-  a.dynamic_lds = p->reduce_lds;   // read by the read-only pass alone; the accumulating passes set their own
   a.xcd_run = p->offgrid ? p->xcd_write_offgrid : p->xcd_write;
   a.scale = scale;
   a.write_on_overflow = 0;
@@ -745,44 +743,10 @@ RG_API int rg_scale_cast(rg_plan* p, float scale, void* stream) {
   return RG_OK;
 }
 
-// Times `launch` (one launch of a pass on `s`) under each candidate setting: three interleaved rounds of one warm-up
-// and two timed launches, each candidate keeping its fastest round, so that a clock ramp or a neighbour's burst does
-// not pick the winner.  Returns the index of the candidate to use: 0 (the setting in use) unless another is more
-// than 1 % faster.
-template <typename Launch>
-static hipError_t fastest_candidate(int n, hipStream_t s, hipEvent_t e0, hipEvent_t e1, Launch launch, int* best_out) {
-  float fastest[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-  hipError_t err = hipSuccess;
-  for (int round = 0; round < 3 && err == hipSuccess; ++round) {
-    for (int k = 0; k < n && err == hipSuccess; ++k) {
-      err = launch(k);                                              // warm-up
-      if (err == hipSuccess) err = hipEventRecord(e0, s);
-      for (int rep = 0; rep < 2 && err == hipSuccess; ++rep) err = launch(k);
-      if (err == hipSuccess) err = hipEventRecord(e1, s);
-      if (err == hipSuccess) err = hipEventSynchronize(e1);
-      float ms = 0.0f;
-      if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
-      if (err == hipSuccess && (fastest[k] == 0.0f || ms < fastest[k])) fastest[k] = ms;
-    }
-  }
-  int best = 0;
-  float best_ms = fastest[0] * 0.99f;
-  for (int k = 1; k < n && err == hipSuccess; ++k) {
-    if (fastest[k] > 0.0f && fastest[k] < best_ms) {
-      best_ms = fastest[k];
-      best = k;
-    }
-  }
-  *best_out = best;
-  return err;
-}
-
 RG_API int rg_plan_tune(rg_plan* p, void* stream) {
-  const int rc = check_plan(p, kNeedSrc, "rg_plan_tune");
+  const int rc = check_plan(p, kNeedSrc | kNeedDst, "rg_plan_tune");
   if (rc != RG_OK) return rc;
-  if (p->n_chunks == 0) return RG_OK;
-  bool has_dst = true;
-  for (const TensorDesc& t : p->host_tensors) has_dst = has_dst && (t.numel == 0 || t.dst != nullptr);
+  if (p->all_in_place || p->n_chunks == 0) return RG_OK;   // nothing that could be run without changing the data
   DeviceGuard guard(p->device);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -791,58 +755,44 @@ RG_API int rg_plan_tune(rg_plan* p, void* stream) {
     (void)hipEventDestroy(e0);
     return hip_fail(hipGetLastError(), "hipEventCreate");
   }
+  // Which order suits a plan depends on how its tensors lie in memory (packed into one bucket or scattered,
+  // on or off each other's line grid) in ways no simple rule captured: measured, the best order differed by up
+  // to 4 % of a pass between plans of the same sizes.
+  // Candidates are timed in turn, three rounds, and each keeps its fastest round, so that a clock ramp or a
+  // neighbour's burst does not pick the winner; the order in use is only given up for a gain above 1 %.
+  const int current = p->offgrid ? p->xcd_write_offgrid : p->xcd_write;
+  int candidates[5] = {current, 0, 64, 256, -1};
+  float fastest[5] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
   hipError_t err = hipSuccess;
-  // The read-only pass: five or all eight blocks resident per compute unit.  The faster one differs from GPU to GPU
-  // (see kReducePassLdsBytes); the pass writes nothing but its partial sums, so any plan with sources can be measured.
-  if (p->streaming) {
-    const unsigned current = p->reduce_lds != 0 ? p->reduce_lds : kReducePassLdsBytes;
-    const unsigned candidates[2] = {current, current == kNoLdsCap ? kReducePassLdsBytes : kNoLdsCap};
-    int best = 0;
-    err = fastest_candidate(2, s, e0, e1, [&](int k) {
-      PassArgs a = pass_args(p, 1.0f);
-      a.xcd_run = p->xcd_reduce;
-      a.dynamic_lds = candidates[k];
-      return launch_pass(kModeReduce, a, true, s);
-    }, &best);
-    if (err == hipSuccess) p->reduce_lds = candidates[best];
-    p->sums_describe_dst = false;
-  }
-  // The writing passes: which order suits a plan depends on how its tensors lie in memory (packed into one bucket or
-  // scattered, on or off each other's line grid) in ways no simple rule captured: measured, the best order differed
-  // by up to 4 % of a pass between plans of the same sizes.  Needs destinations it may overwrite.
-  if (err == hipSuccess && has_dst && !p->all_in_place) {
-    const int current = p->offgrid ? p->xcd_write_offgrid : p->xcd_write;
-    int candidates[5] = {current, 0, 64, 256, -1};
-    int n = 1;
-    for (int k = 1; k < 5; ++k)
-      if (candidates[k] != current) candidates[n++] = candidates[k];
-    int best = 0;
-    err = fastest_candidate(n, s, e0, e1, [&](int k) {
+  for (int round = 0; round < 3 && err == hipSuccess; ++round) {
+    for (int k = 0; k < 5 && err == hipSuccess; ++k) {
+      if (k > 0 && candidates[k] == current) continue;
       PassArgs a = pass_args(p, 1.0f);
       a.xcd_run = candidates[k];
       split_for_write(p, a);
-      return launch_pass(kModeWrite, a, p->streaming, s);
-    }, &best);
-    if (err == hipSuccess) p->xcd_write = p->xcd_write_offgrid = candidates[best];
-    p->sums_describe_dst = false;
+      err = launch_pass(kModeWrite, a, p->streaming, s);           // warm-up
+      if (err == hipSuccess) err = hipEventRecord(e0, s);
+      for (int rep = 0; rep < 2 && err == hipSuccess; ++rep) err = launch_pass(kModeWrite, a, p->streaming, s);
+      if (err == hipSuccess) err = hipEventRecord(e1, s);
+      if (err == hipSuccess) err = hipEventSynchronize(e1);
+      float ms = 0.0f;
+      if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+      if (err == hipSuccess && (fastest[k] == 0.0f || ms < fastest[k])) fastest[k] = ms;
+    }
+  }
+  int best = current;
+  float best_ms = fastest[0] * 0.99f;
+  for (int k = 1; k < 5 && err == hipSuccess; ++k) {
+    if (fastest[k] > 0.0f && fastest[k] < best_ms) {
+      best_ms = fastest[k];
+      best = candidates[k];
+    }
   }
   (void)hipEventDestroy(e0);
   (void)hipEventDestroy(e1);
   if (err != hipSuccess) return hip_fail(err, "rg_plan_tune");
-  return RG_OK;
-}
-
-RG_API int rg_plan_read_residency(const rg_plan* p) {
-  if (p == nullptr) return -1;
-  return (p->reduce_lds != 0 ? p->reduce_lds : kReducePassLdsBytes) == kNoLdsCap ? 8 : 5;
-}
-
-RG_API int rg_plan_set_read_residency(rg_plan* p, int blocks) {
-  if (p == nullptr || (blocks != 5 && blocks != 8)) {
-    set_error("rg_plan_set_read_residency: bad arguments (blocks %d: 5 or 8)", blocks);
-    return RG_EINVAL;
-  }
-  p->reduce_lds = blocks == 8 ? kNoLdsCap : kReducePassLdsBytes;
+  p->xcd_write = p->xcd_write_offgrid = best;
+  p->sums_describe_dst = false;
   return RG_OK;
 }
 

@@ -92,12 +92,7 @@ __host__ __device__ inline int head_elems(uintptr_t addr, unsigned align, unsign
 }
 constexpr int64_t kChunkQuantum = 2048;    // chunk sizes are multiples of this many elements
 constexpr int64_t kMaxChunkElems = 1 << 20;
-// Dynamic LDS of the streaming read-only pass: unused, it only caps the blocks resident per compute unit (160 KiB):
-// 32768 -> five blocks of 256 threads instead of the eight that fit.  Which of the two is faster depends on the GPU
-// the process runs on, not on the plan (measured on MI355X boxes of one pool: on some, five blocks 92.8 % of peak and
-// eight 89.3 % on 5 GB of fp16; on others 90.4 % and 92.4 %), so rg_plan_tune measures it and the cap is the default.
-constexpr unsigned kReducePassLdsBytes = 32768;
-constexpr unsigned kNoLdsCap = 16;                // a PassArgs::dynamic_lds that caps nothing
+constexpr unsigned kReducePassLdsBytes = 32768;   // dynamic LDS of the streaming read-only pass: 5 resident blocks per compute unit
 // rg_accumulate's pass reads more than it writes (source and old destination in, destination out) and, like the
 // read-only pass, runs faster with fewer blocks resident per compute unit (measured on MI355X, streaming sizes):
 // with 16 bytes loaded from each side per lane and step (both sides equally wide) ten blocks of 128 threads instead
@@ -154,8 +149,7 @@ struct PassArgs {
   int32_t only_if_clipped;       // with `result`: the whole launch does nothing unless result->clipped is set
   int32_t src_is_dst;            // read the destination instead of the record's source (in-place rescale)
   int32_t chunks_per_block;      // launch_gated_pass only: consecutive chunks one block walks through
-  uint32_t dynamic_lds;          // host side only: unused dynamic LDS that caps the resident blocks of a read-only or
-                                 // accumulating pass (0: the mode's default; kNoLdsCap: none)
+  uint32_t dynamic_lds;          // host side only: unused dynamic LDS that caps the resident blocks (0: the mode's default)
 };
 
 struct ReduceArgs {

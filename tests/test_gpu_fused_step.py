@@ -230,50 +230,6 @@ def test_every_write_order_gives_the_oracles_bits(order):
     plan.close()
 
 
-@pytest.mark.parametrize("blocks", [5, 8])
-def test_read_pass_residency_changes_only_the_time(blocks):
-    """How many blocks of the streaming read-only pass a compute unit holds (``rg_plan_set_read_residency``, what
-    ``rg_plan_tune`` measures) is a matter of time alone: flag, norms and the decision are the oracle's either way."""
-    g = torch.Generator().manual_seed(78)
-    grads = [(torch.randn(n, generator=g) * 8).to(torch.float16) for n in (100003, 5, 16384, 40000, 1, 262147)]
-    srcs = place_in_arena(grads, DEV, 1, 3)
-    dsts = [torch.full((t.numel(),), 3.0, device=DEV) for t in grads]
-    plan = TensorPlan(srcs, dsts, chunk_elems=4096)
-    plan.plan.set_streaming(1)                      # the cap only exists in the streaming form of the pass
-    assert plan.read_residency() == 5               # the default
-    plan.set_read_residency(blocks)
-    assert plan.read_residency() == blocks
-    plan.fused_step(0.125, 0.5)
-    res, tn = plan.result(), plan.tensor_norms()
-    want = oracle.fused_step(grads, ["f32"] * len(grads), 0.125, 0.5)
-    assert res.overflow == want.overflow and res.clipped == 1
-    assert math.isclose(res.norm, want.norm, rel_tol=1e-6)
-    for got, w in zip(tn, want.tensor_norms):
-        assert math.isclose(got, w, rel_tol=1e-6, abs_tol=1e-30)
-    offs, _ = oracle.bucket_layout([t.numel() for t in grads], ["f32"] * len(grads))
-    for d, o in zip(dsts, offs):
-        assert_bits_equal(d.cpu(), want.buckets["f32"][o:o + d.numel()], "written bits")
-    plan.grad_norm()
-    assert math.isclose(plan.result().norm, oracle.grad_global_l2_norm(grads), rel_tol=1e-6)
-    with pytest.raises(ValueError, match="blocks"):
-        plan.set_read_residency(6)
-    plan.close()
-
-
-def test_tune_measures_a_plan_without_destinations():
-    """A plan that only reads (``rg_grad_norm``) can be tuned too: only the read pass is measured."""
-    g = torch.Generator().manual_seed(79)
-    cpu = [torch.randn(n, generator=g) for n in (70001, 3, 300000)]
-    srcs = [t.to(DEV) for t in cpu]
-    plan = TensorPlan(srcs, [None] * len(srcs))
-    plan.plan.set_streaming(1)
-    plan.tune()
-    assert plan.read_residency() in (5, 8)
-    plan.grad_norm()
-    assert math.isclose(plan.result().norm, oracle.grad_global_l2_norm(cpu), rel_tol=1e-6)
-    plan.close()
-
-
 def test_set_write_order_rejects_values_outside_its_range():
     t = torch.zeros(4096, device=DEV)
     plan = TensorPlan([t], [torch.zeros_like(t)])
