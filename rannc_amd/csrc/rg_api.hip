@@ -57,6 +57,7 @@ struct rg_plan {
   bool all_in_place = false;         // every tensor with elements has dst == src (and so one dtype)
   char* dst_range = nullptr;         // the destinations, in plan order, lie back to back: one range of dst_range_bytes
   int64_t dst_range_bytes = 0;       //   (a gradient bucket's views); null when they do not
+  int64_t dst_bytes = 0;             // bytes of all destinations
 
   // one device allocation, carved up
   char* dev_base = nullptr;
@@ -106,11 +107,13 @@ static void fill_chunk_records(rg_plan* p, ChunkRec* out) {
   p->all_in_place = true;
   p->dst_range = nullptr;
   p->dst_range_bytes = 0;
+  p->dst_bytes = 0;
   bool back_to_back = true;
   for (int i = 0; i < p->n_tensors; ++i) {
     const TensorDesc& t = p->host_tensors[(size_t)i];
     if (t.numel > 0 && (t.dst == nullptr || t.dst != t.src)) p->all_in_place = false;
     const int ss = elem_size(t.src_dtype), ds = elem_size(t.dst_dtype);
+    if (t.dst != nullptr) p->dst_bytes += t.numel * ds;
     if (t.numel > 0 && back_to_back) {
       char* d = static_cast<char*>(t.dst);
       if (d == nullptr || (p->dst_range != nullptr && d != p->dst_range + p->dst_range_bytes)) {
@@ -995,6 +998,12 @@ RG_API int rg_zero(rg_plan* p, void* stream) {
   // (measured on MI355X: BERT-large's bucket 83 % of peak round robin, 91.5 % with runs of 64 tiles, 90.6 % with
   // runs of 256, 86 % with contiguous eighths; the ResNet's 83.7 / 87.2 / 87.8 / 82.5 %).
   a.xcd_run = kZeroXcdRun;
+  // Scattered destinations of streaming size: the flat fill's pacing in small.  A wavefront here first fetches its
+  // chunk record, which spaces the stores already; holding it another 0.1 us pays from about 1.5 GiB (64 MiB
+  // tensors, % of peak without / with: 1 GiB 93.8 / 92.9, 1.5 GiB 91.8 / 92.8, 2 GiB 91.4 / 93.2, 4 GiB 89.6 / 92.6,
+  // 8 GiB 89.7 / 92.5; the 775 fp16 gradients of a 2.5e9-parameter stage 88.9 -> 92.9 %) and costs 2-4 points
+  // below 1 GiB.
+  if (p->streaming && p->dst_bytes >= kZeroDelayMinBytes) a.zero_delay_ticks = fill_delay_ticks(kZeroDelayNs);
   RG_HIP(launch_pass(kModeWrite, a, p->streaming, reinterpret_cast<hipStream_t>(stream)));
   return RG_OK;
 }

@@ -101,6 +101,8 @@ constexpr unsigned kReducePassLdsBytes = 32768;   // dynamic LDS of the streamin
 // sums (rg_unscale_accumulate) holds twelve blocks by its register count already (ten gain on flat same-width data
 // but lose on the ResNet's many small tensors); plain writing passes lose from the first block taken away.
 constexpr int kZeroXcdRun = 64;                      // rg_zero: tiles of a run one XCD fills (see rg_zero)
+constexpr int kZeroDelayNs = 100;                    // rg_zero through the table, large plans: wall-clock hold before a tile's stores
+constexpr int64_t kZeroDelayMinBytes = (int64_t)1536 << 20;
 constexpr unsigned kAccSameWidthLdsBytes = 16384;   // 10 resident blocks
 constexpr unsigned kAccMixedWidthLdsBytes = 13600;  // 12 resident blocks
 constexpr int64_t kMinWriteTileElems = 256;    // bounds the per-tile partial storage of a plan
@@ -145,6 +147,7 @@ struct PassArgs {
   const float* scale_dev;        // non-null: the kernels read the scale from device memory instead of `scale`
   int32_t write_on_overflow;
   int32_t zero_fill;             // write pass: ignore the sources, store zeros
+  int32_t zero_delay_ticks;      // ... after holding each wavefront for this many ticks of the wall clock (0: none)
   int32_t norm_of_source;        // reduce pass: measure the source as stored (no rounding to dst)
   int32_t only_if_clipped;       // with `result`: the whole launch does nothing unless result->clipped is set
   int32_t src_is_dst;            // read the destination instead of the record's source (in-place rescale)
@@ -180,6 +183,7 @@ hipError_t launch_decide(const ReduceArgs& a, hipStream_t stream);
 hipError_t launch_fill_zero(void* dst, int64_t nbytes, hipStream_t stream);
 // Ticks of the current device's wall clock that a wavefront of a large flat fill waits before it stores (0: unknown rate).
 int fill_delay_ticks();
+int fill_delay_ticks(int ns);   // the same clock, another delay
 
 void set_error(const char* fmt, ...);
 

@@ -296,6 +296,10 @@ __device__ __forceinline__ void pass_block(const PassArgs& a, unsigned bid, floa
         else process_chunk<RG_BF16, RG_BF16, kModeReduce, NT, T>(dp, dp, len, 1.0f, 1.0f, false, acc);
       }
     } else if (MODE & kModeWrite) {
+      if (NT && a.zero_delay_ticks > 0) {   // see rg_zero
+        const uint64_t t_end = wall_clock64() + (uint64_t)a.zero_delay_ticks;
+        while (wall_clock64() < t_end) __builtin_amdgcn_s_sleep(1);
+      }
       zero_range<NT, T, PEEL>(dp, len * (rec.dst_dtype == RG_F32 ? 4 : 2));
     }
   } else {
@@ -717,6 +721,11 @@ hipError_t launch_decide(const ReduceArgs& a, hipStream_t stream) {
 #endif
 constexpr int kFillDelayNs = RG_FILL_DELAY_NS;
 constexpr int kMaxDevices = 64;
+int fill_delay_ticks(int ns) {
+  const int t = fill_delay_ticks();
+  return t > 0 ? (int)(((int64_t)t * ns + kFillDelayNs / 2) / kFillDelayNs) : 0;
+}
+
 int fill_delay_ticks() {
   static std::atomic<int> cached[kMaxDevices];   // 0: not asked yet; -1: unknown rate
   int dev = 0;

@@ -107,6 +107,21 @@ def test_zero_over_back_to_back_destinations_and_after_they_move_apart():
     plan.close()
 
 
+def test_zero_of_scattered_destinations_of_a_streaming_size():
+    """Above 1.5 GiB the table-driven clear holds every tile's wavefronts for a moment before they store (pacing);
+    the bytes it writes are the same: every destination zero, every gap between them untouched."""
+    k, n, gap = 26, (16 << 20) + 5, 37                       # 26 tensors of 64 MiB + 20 B, 148-byte gaps: 1.63 GiB
+    arena = torch.full((k * (n + gap) + gap,), 3.0, dtype=torch.float32, device=DEV)
+    dsts = [arena[gap + i * (n + gap):gap + i * (n + gap) + n] for i in range(k)]
+    plan = TensorPlan([None] * k, dsts)
+    plan.zero()
+    torch.cuda.synchronize()
+    assert int((arena == 0).sum()) == k * n
+    assert all(bool((d == 0).all()) for d in dsts)
+    assert int((arena == 3.0).sum()) == (k + 1) * gap
+    plan.close()
+
+
 @pytest.mark.parametrize("dst_name", ["f32", "f16", "bf16"])
 def test_zero_fills_only_the_destinations(dst_name):
     ddt = TORCH_DTYPE[dst_name]
